@@ -1,0 +1,161 @@
+/*
+ * lvx.h - C ABI of the MI355X (gfx950) cross-attention hot path of LV-XAttn.
+ *
+ * One shared library (liblvx.so) built by hipcc; a Python, C or C++ host binds
+ * these symbols directly (ctypes / dlopen).  Nothing here uses a torch type.
+ *
+ * Conventions
+ *   - every data pointer is a DEVICE pointer owned by the caller; the library
+ *     allocates nothing, keeps no pointer after a call returns and never
+ *     synchronises: all work is queued on `stream` (a hipStream_t, NULL = the
+ *     default stream);
+ *   - 16-bit tensors are bf16; strides are in ELEMENTS, the last (head_dim)
+ *     stride is 1, every other stride is a multiple of 8 and every base pointer
+ *     is 16-byte aligned;
+ *   - q-like tensors are indexed [batch, q_head, text_row, d], kv-like tensors
+ *     [batch, kv_head, visual_token, d] with Hq % Hkv == 0; q head h reads kv
+ *     head h / (Hq/Hkv) (the order lv_xattn/attn.py:271-277 expands to);
+ *   - LSE / delta are fp32 [B*Hq, Lq] contiguous, natural-log LSE of
+ *     scale*q.k (lv_xattn/attn.py:265-268);
+ *   - [row_begin, row_begin+row_count) selects the text rows one call works on:
+ *     one query block of one round, or all of them at once;
+ *   - return value: 0 = queued; negative = argument rejected on the host before
+ *     anything was launched (LVX_ERR_*); positive = hipError_t of the launch.
+ *     Nothing throws or aborts.  Calls are re-entrant.
+ */
+#ifndef LVX_H
+#define LVX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LVX_VERSION 100
+
+#define LVX_OK 0
+#define LVX_ERR_NULL (-1)        /* a required pointer is NULL */
+#define LVX_ERR_ALIGN (-2)       /* pointer not 16-byte aligned / stride not a multiple of 8 */
+#define LVX_ERR_SHAPE (-3)       /* non-positive or inconsistent sizes, bad row window */
+#define LVX_ERR_HEAD_DIM (-4)    /* head_dim other than 128 */
+#define LVX_ERR_DTYPE (-5)       /* dtype other than LVX_BF16 */
+#define LVX_ERR_SCALE (-6)       /* scale must be finite and > 0 */
+#define LVX_ERR_WORKSPACE (-7)   /* workspace missing or too small */
+#define LVX_ERR_UNSUPPORTED (-8) /* valid request this build does not implement */
+
+#define LVX_BF16 1
+
+/* Sizes shared by the attention entry points. */
+typedef struct lvx_attn_shape {
+    int32_t B, Hq, Hkv, D;
+    int32_t Lq;              /* text rows per sample (padded length)        */
+    int32_t Lkv;             /* visual tokens per sample (padded length)    */
+    int32_t dtype;           /* LVX_BF16                                    */
+    float scale;             /* softmax scale, applied before the mask      */
+    const int32_t* kv_len;   /* [B] valid visual tokens per sample, or NULL */
+    const int32_t* kv_start; /* [B, Lq] first visible token per text row, or NULL */
+    const int32_t* kv_end;   /* [B, Lq] one past the last visible token (both or neither) */
+} lvx_attn_shape;
+
+/* A 4-d tensor with unit last stride. */
+typedef struct lvx_tensor {
+    void* ptr;
+    int64_t stride_b, stride_h, stride_s;
+} lvx_tensor;
+
+int lvx_version(void);
+const char* lvx_strerror(int code);
+
+/*
+ * Flash cross-attention forward of the selected text rows against the whole
+ * local K/V shard: O (bf16, normalised) and LSE.  Rows that see no key get
+ * O = 0 and LSE = -inf.  Replaces the `_fwd_kernel` launch of one round
+ * (lv_xattn/attn.py:140-268, launched at :390-400) and the per-round KV head
+ * expansion (:271-277, :392-393), which happens in-kernel here.
+ * kv_splits > 1 cuts the shard into that many key ranges computed by separate
+ * work-groups and folded before return; it needs a workspace of
+ * lvx_fwd_workspace_bytes(shape, row_count, kv_splits) bytes.
+ */
+int lvx_fwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
+            const lvx_tensor* v, const lvx_tensor* o, float* lse,
+            int32_t row_begin, int32_t row_count, int32_t kv_splits,
+            void* workspace, size_t workspace_bytes, void* stream);
+
+size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* shape, int32_t row_count, int32_t kv_splits);
+
+/*
+ * Rescale-merge: folds a partial (o_part, l_part) over one key set into the
+ * travelling accumulator (o_acc, l_acc) of the same rows, in place:
+ *   L' = ln(e^La + e^Lb),  O' = Oa e^(La-L') + Ob e^(Lb-L').
+ * Replaces `_rescale_kernel` (lv_xattn/attn.py:37-110, launched at :405-419),
+ * evaluated with the maximum subtracted; (-inf, -inf) stays (0, -inf).
+ */
+int lvx_merge(const lvx_attn_shape* shape, const lvx_tensor* o_acc, float* l_acc,
+              const lvx_tensor* o_part, const float* l_part,
+              int32_t row_begin, int32_t row_count, void* stream);
+
+/*
+ * delta[b*Hq+h, row] = sum_d O * dO.  Replaces `_bwd_preprocess_do_o_dot`
+ * (lv_xattn/flash_attn_kernels.py:287-329, launched at :926-942).
+ */
+int lvx_bwd_preprocess(const lvx_attn_shape* shape, const lvx_tensor* o, const lvx_tensor* dout,
+                       float* delta, int32_t row_begin, int32_t row_count, void* stream);
+
+/*
+ * Backward of the selected text rows against the whole local shard, from the
+ * saved (finally merged) LSE and delta.  Replaces `_bwd_kernel`
+ * (lv_xattn/flash_attn_kernels.py:364-640, 677-819; launcher :904-1020) and the
+ * host-side `dk += dk_delta; dv += dv_delta` of lv_xattn/attn.py:523-524.
+ *   dq_acc : fp32 [B, Hq, Lq, D] contiguous; contributions are ADDED (atomic),
+ *            the caller zeroes it once before the first round;
+ *   dk, dv : at Hkv heads (the group sum is taken in registers);
+ *            dkv_accumulate == 0: bf16 tensors, overwritten;
+ *            dkv_accumulate == 1: fp32 tensors of the same indexing, added to.
+ */
+int lvx_bwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
+            const lvx_tensor* v, const lvx_tensor* dout, const float* lse, const float* delta,
+            float* dq_acc, const lvx_tensor* dk, const lvx_tensor* dv, int32_t dkv_accumulate,
+            int32_t row_begin, int32_t row_count, void* stream);
+
+/*
+ * dst(bf16, strided) = src(fp32, [B, H, L, D] contiguous): the final rounding of
+ * an fp32 accumulator (the `dq.copy_(dq_accum)` of flash_attn_kernels.py:1020).
+ */
+int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L,
+                      int32_t D, void* stream);
+
+/*
+ * K/V recompute from the shared visual hidden states:
+ *   K[M, N] = X[M, Dm] * W_k,   V[M, N] = X[M, Dm] * W_v      (bf16 in, fp32 accumulate)
+ * with M = B*Lkv rows and N = Hkv*D columns, so K/V land in [B, Lkv, Hkv, D]
+ * memory order.  Replaces the k_proj / v_proj nn.Linear calls inside `project`
+ * (test_llama3.py:395-398) run in forward and again in backward (:197, :235).
+ * w_in_major != 0: W is [Dm, N] row-major;  w_in_major == 0: W is [N, Dm]
+ * row-major (torch.nn.Linear.weight).  ld* are row strides in elements.
+ */
+int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw,
+                int32_t w_in_major, void* k_out, void* v_out, int64_t ldkv,
+                int32_t M, int32_t Dm, int32_t N, void* stream);
+
+/*
+ * dX[M, Dm] = dK[M, N] * W_k^T + dV[M, N] * W_v^T  (no counterpart in the
+ * reference, whose wrapper drops this gradient: test_llama3.py:243).
+ */
+int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v,
+               int64_t ldw, int32_t w_in_major, void* dx, int64_t lddx,
+               int32_t M, int32_t Dm, int32_t N, void* stream);
+
+/*
+ * dW_k = X^T dK, dW_v = X^T dV in the layout of W (see w_in_major); the weight
+ * gradients the recompute path needs to train the projections.
+ */
+int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_t lddkv,
+              void* dw_k, void* dw_v, int64_t ldw, int32_t w_in_major,
+              int32_t M, int32_t Dm, int32_t N, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LVX_H */

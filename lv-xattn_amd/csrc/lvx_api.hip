@@ -1,0 +1,336 @@
+// C-ABI layer: argument validation on the host (nothing is launched when a
+// check fails), translation to the internal launch parameters, error strings.
+#include "../../include/lvx.h"
+#include "lvx_kernels.hpp"
+
+#include <cmath>
+
+using namespace lvx;
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_tensor(const lvx_tensor* t) {
+    if (!t || !t->ptr) return LVX_ERR_NULL;
+    if (!aligned16(t->ptr)) return LVX_ERR_ALIGN;
+    if ((t->stride_b % 8) || (t->stride_h % 8) || (t->stride_s % 8)) return LVX_ERR_ALIGN;
+    if (t->stride_s <= 0) return LVX_ERR_SHAPE;
+    return LVX_OK;
+}
+
+int check_shape(const lvx_attn_shape* s) {
+    if (!s) return LVX_ERR_NULL;
+    if (s->dtype != LVX_BF16) return LVX_ERR_DTYPE;
+    if (s->D != 128) return LVX_ERR_HEAD_DIM;
+    if (s->B <= 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Lq <= 0 || s->Lkv <= 0) return LVX_ERR_SHAPE;
+    if (s->Hq % s->Hkv) return LVX_ERR_SHAPE;
+    if (!(s->scale > 0.f) || !std::isfinite(s->scale)) return LVX_ERR_SCALE;
+    if ((s->kv_start == nullptr) != (s->kv_end == nullptr)) return LVX_ERR_NULL;
+    return LVX_OK;
+}
+
+int check_rows(const lvx_attn_shape* s, int32_t row_begin, int32_t row_count) {
+    if (row_begin < 0 || row_count < 0 || (int64_t)row_begin + row_count > s->Lq) return LVX_ERR_SHAPE;
+    return LVX_OK;
+}
+
+inline Strides3 st3(const lvx_tensor* t) { return Strides3{t->stride_b, t->stride_h, t->stride_s}; }
+
+inline int gcd(int a, int b) { return b ? gcd(b, a % b) : a; }
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr int FWD_BN = 64;
+constexpr int MAX_SPLITS = 16;
+
+#define LVX_TRY(expr)            \
+    do {                         \
+        int rc_ = (expr);        \
+        if (rc_ != LVX_OK) return rc_; \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int lvx_version(void) { return LVX_VERSION; }
+
+const char* lvx_strerror(int code) {
+    switch (code) {
+        case LVX_OK: return "ok";
+        case LVX_ERR_NULL: return "a required pointer is NULL";
+        case LVX_ERR_ALIGN: return "pointer not 16-byte aligned or stride not a multiple of 8 elements";
+        case LVX_ERR_SHAPE: return "bad sizes or row window";
+        case LVX_ERR_HEAD_DIM: return "head_dim must be 128";
+        case LVX_ERR_DTYPE: return "dtype must be LVX_BF16";
+        case LVX_ERR_SCALE: return "scale must be finite and > 0";
+        case LVX_ERR_WORKSPACE: return "workspace missing or too small";
+        case LVX_ERR_UNSUPPORTED: return "not supported by this build";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown lvx error";
+}
+
+size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count, int32_t kv_splits) {
+    if (!s || kv_splits <= 1 || row_count <= 0) return 0;
+    const size_t rows = (size_t)s->B * s->Hq * row_count;
+    return (size_t)kv_splits * rows * (s->D * sizeof(uint16_t) + sizeof(float));
+}
+
+int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+            const lvx_tensor* o, float* lse, int32_t row_begin, int32_t row_count, int32_t kv_splits,
+            void* workspace, size_t workspace_bytes, void* stream) {
+    LVX_TRY(check_shape(s));
+    LVX_TRY(check_tensor(q));
+    LVX_TRY(check_tensor(k));
+    LVX_TRY(check_tensor(v));
+    LVX_TRY(check_tensor(o));
+    if (!lse) return LVX_ERR_NULL;
+    LVX_TRY(check_rows(s, row_begin, row_count));
+    if (kv_splits < 1 || kv_splits > MAX_SPLITS) return LVX_ERR_SHAPE;
+    if (row_count == 0) return LVX_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    FwdParams p{};
+    p.q = static_cast<const uint16_t*>(q->ptr);
+    p.k = static_cast<const uint16_t*>(k->ptr);
+    p.v = static_cast<const uint16_t*>(v->ptr);
+    p.qs = st3(q); p.ks = st3(k); p.vs = st3(v);
+    p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
+    p.B = s->B; p.Hq = s->Hq; p.Hkv = s->Hkv; p.Lq = s->Lq; p.Lkv = s->Lkv;
+    p.G = s->Hq / s->Hkv;
+    p.HG = gcd(p.G, 4);
+    p.RS = 4 / p.HG;
+    p.row_begin = row_begin; p.row_end = row_begin + row_count;
+    p.n_row_tiles = (row_count + 32 * p.RS - 1) / (32 * p.RS);
+    p.n_head_groups = s->Hq / p.HG;
+    p.scale = s->scale; p.scale_log2e = s->scale * LOG2E;
+
+    int nsplit = kv_splits;
+    int split_len = ((s->Lkv + nsplit - 1) / nsplit + FWD_BN - 1) / FWD_BN * FWD_BN;
+    nsplit = (s->Lkv + split_len - 1) / split_len;
+    p.nsplit = nsplit;
+    p.split_len = split_len;
+    p.total_wg = s->B * p.n_head_groups * nsplit * p.n_row_tiles;
+
+    if (nsplit == 1) {
+        p.o = static_cast<uint16_t*>(o->ptr);
+        p.os = st3(o);
+        p.lse = lse;
+        p.lse_bh_stride = s->Lq;
+        return static_cast<int>(launch_fwd(p, s->kv_start != nullptr, st));
+    }
+
+    // key splits: partials [split][B*Hq][row_count][D] + LSE [split][B*Hq][row_count]
+    const size_t need = lvx_fwd_workspace_bytes(s, row_count, nsplit);
+    if (!workspace || workspace_bytes < need) return LVX_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return LVX_ERR_ALIGN;
+    const int64_t rows = (int64_t)s->B * s->Hq * row_count;
+    uint16_t* o_ws = static_cast<uint16_t*>(workspace);
+    float* l_ws = reinterpret_cast<float*>(o_ws + (int64_t)nsplit * rows * s->D);
+    // the kernel indexes partials by absolute row: bias the bases by -row_begin
+    p.o = o_ws - (int64_t)row_begin * s->D;
+    p.os = Strides3{(int64_t)s->Hq * row_count * s->D, (int64_t)row_count * s->D, s->D};
+    p.o_split_stride = rows * s->D;
+    p.lse = l_ws - row_begin;
+    p.lse_bh_stride = row_count;
+    p.lse_split_stride = rows;
+    hipError_t e = launch_fwd(p, s->kv_start != nullptr, st);
+    if (e != hipSuccess) return static_cast<int>(e);
+
+    MergeParams m{};
+    m.o_acc = static_cast<uint16_t*>(o->ptr);
+    m.l_acc = lse;
+    m.o_part = p.o;
+    m.l_part = p.lse;
+    m.oa = st3(o);
+    m.op = p.os;
+    m.o_part_stride = p.o_split_stride;
+    m.l_part_stride = p.lse_split_stride;
+    m.l_acc_bh = s->Lq;
+    m.l_part_bh = row_count;
+    m.nparts = nsplit;
+    m.use_acc = 0;
+    m.B = s->B; m.Hq = s->Hq; m.Lq = s->Lq;
+    m.row_begin = row_begin; m.row_end = row_begin + row_count;
+    return static_cast<int>(launch_merge(m, st));
+}
+
+int lvx_merge(const lvx_attn_shape* s, const lvx_tensor* o_acc, float* l_acc, const lvx_tensor* o_part,
+              const float* l_part, int32_t row_begin, int32_t row_count, void* stream) {
+    LVX_TRY(check_shape(s));
+    LVX_TRY(check_tensor(o_acc));
+    LVX_TRY(check_tensor(o_part));
+    if (!l_acc || !l_part) return LVX_ERR_NULL;
+    LVX_TRY(check_rows(s, row_begin, row_count));
+    MergeParams m{};
+    m.o_acc = static_cast<uint16_t*>(o_acc->ptr);
+    m.l_acc = l_acc;
+    m.o_part = static_cast<const uint16_t*>(o_part->ptr);
+    m.l_part = l_part;
+    m.oa = st3(o_acc);
+    m.op = st3(o_part);
+    m.l_acc_bh = s->Lq;
+    m.l_part_bh = s->Lq;
+    m.nparts = 1;
+    m.use_acc = 1;
+    m.B = s->B; m.Hq = s->Hq; m.Lq = s->Lq;
+    m.row_begin = row_begin; m.row_end = row_begin + row_count;
+    return static_cast<int>(launch_merge(m, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_tensor* dout, float* delta,
+                       int32_t row_begin, int32_t row_count, void* stream) {
+    LVX_TRY(check_shape(s));
+    LVX_TRY(check_tensor(o));
+    LVX_TRY(check_tensor(dout));
+    if (!delta) return LVX_ERR_NULL;
+    LVX_TRY(check_rows(s, row_begin, row_count));
+    PreParams p{};
+    p.o = static_cast<const uint16_t*>(o->ptr);
+    p.dout = static_cast<const uint16_t*>(dout->ptr);
+    p.delta = delta;
+    p.os = st3(o); p.ds = st3(dout);
+    p.B = s->B; p.Hq = s->Hq; p.Lq = s->Lq;
+    p.row_begin = row_begin; p.row_end = row_begin + row_count;
+    return static_cast<int>(launch_preprocess(p, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+            const lvx_tensor* dout, const float* lse, const float* delta, float* dq_acc,
+            const lvx_tensor* dk, const lvx_tensor* dv, int32_t dkv_accumulate,
+            int32_t row_begin, int32_t row_count, void* stream) {
+    LVX_TRY(check_shape(s));
+    LVX_TRY(check_tensor(q));
+    LVX_TRY(check_tensor(k));
+    LVX_TRY(check_tensor(v));
+    LVX_TRY(check_tensor(dout));
+    LVX_TRY(check_tensor(dk));
+    LVX_TRY(check_tensor(dv));
+    if (!lse || !delta || !dq_acc) return LVX_ERR_NULL;
+    if (!aligned16(dq_acc)) return LVX_ERR_ALIGN;
+    if (dkv_accumulate != 0 && dkv_accumulate != 1) return LVX_ERR_SHAPE;
+    LVX_TRY(check_rows(s, row_begin, row_count));
+    BwdParams p{};
+    p.q = static_cast<const uint16_t*>(q->ptr);
+    p.k = static_cast<const uint16_t*>(k->ptr);
+    p.v = static_cast<const uint16_t*>(v->ptr);
+    p.dout = static_cast<const uint16_t*>(dout->ptr);
+    p.lse = lse; p.delta = delta; p.dq_acc = dq_acc;
+    p.dk = dk->ptr; p.dv = dv->ptr;
+    p.qs = st3(q); p.ks = st3(k); p.vs = st3(v); p.dos = st3(dout); p.dks = st3(dk); p.dvs = st3(dv);
+    p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
+    p.B = s->B; p.Hq = s->Hq; p.Hkv = s->Hkv; p.Lq = s->Lq; p.Lkv = s->Lkv; p.G = s->Hq / s->Hkv;
+    p.row_begin = row_begin; p.row_end = row_begin + row_count;
+    p.n_kv_blocks = (s->Lkv + 127) / 128;
+    p.total_wg = s->B * s->Hkv * p.n_kv_blocks;
+    p.dkv_accumulate = dkv_accumulate;
+    p.scale = s->scale; p.scale_log2e = s->scale * LOG2E;
+    return static_cast<int>(launch_bwd(p, s->kv_start != nullptr, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L, int32_t D,
+                      void* stream) {
+    if (!src) return LVX_ERR_NULL;
+    LVX_TRY(check_tensor(dst));
+    if (!aligned16(src)) return LVX_ERR_ALIGN;
+    if (D != 128) return LVX_ERR_HEAD_DIM;
+    if (B <= 0 || H <= 0 || L <= 0) return LVX_ERR_SHAPE;
+    CastParams p{};
+    p.src = src;
+    p.dst = static_cast<uint16_t*>(dst->ptr);
+    p.ds = st3(dst);
+    p.B = B; p.H = H; p.L = L;
+    return static_cast<int>(launch_cast(p, static_cast<hipStream_t>(stream)));
+}
+
+static int check_gemm_ptr(const void* p, int64_t ld) {
+    if (!p) return LVX_ERR_NULL;
+    if (!aligned16(p) || (ld % 8) != 0) return LVX_ERR_ALIGN;
+    if (ld <= 0) return LVX_ERR_SHAPE;
+    return LVX_OK;
+}
+
+static void fill_grid(GemmParams& g, int M, int N, int nprob) {
+    g.M = M; g.N = N; g.nprob = nprob;
+    g.tiles_m = (M + 127) / 128;
+    g.tiles_n = (N + 127) / 128;
+    g.total_wg = nprob * g.tiles_m * g.tiles_n;
+}
+
+int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
+                void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, void* stream) {
+    LVX_TRY(check_gemm_ptr(x, ldx));
+    LVX_TRY(check_gemm_ptr(w_k, ldw));
+    LVX_TRY(check_gemm_ptr(w_v, ldw));
+    LVX_TRY(check_gemm_ptr(k_out, ldkv));
+    LVX_TRY(check_gemm_ptr(v_out, ldkv));
+    if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
+    if (ldx < Dm || ldkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
+    GemmParams g{};
+    const void* w[2] = {w_k, w_v};
+    void* c[2] = {k_out, v_out};
+    for (int i = 0; i < 2; ++i) {
+        GemmProblem& pr = g.prob[i];
+        pr.A[0] = static_cast<const uint16_t*>(x); pr.lda[0] = ldx;
+        pr.Bm[0] = static_cast<const uint16_t*>(w[i]); pr.ldb[0] = ldw;
+        pr.K[0] = Dm; pr.nseg = 1;
+        pr.C = static_cast<uint16_t*>(c[i]); pr.ldc = ldkv;
+    }
+    fill_grid(g, M, N, 2);
+    return static_cast<int>(launch_gemm(g, false, w_in_major != 0, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v, int64_t ldw,
+               int32_t w_in_major, void* dx, int64_t lddx, int32_t M, int32_t Dm, int32_t N, void* stream) {
+    LVX_TRY(check_gemm_ptr(dk, lddkv));
+    LVX_TRY(check_gemm_ptr(dv, lddkv));
+    LVX_TRY(check_gemm_ptr(w_k, ldw));
+    LVX_TRY(check_gemm_ptr(w_v, ldw));
+    LVX_TRY(check_gemm_ptr(dx, lddx));
+    if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
+    if (lddkv < N || lddx < Dm || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
+    GemmParams g{};
+    GemmProblem& pr = g.prob[0];
+    pr.A[0] = static_cast<const uint16_t*>(dk); pr.A[1] = static_cast<const uint16_t*>(dv);
+    pr.lda[0] = pr.lda[1] = lddkv;
+    pr.Bm[0] = static_cast<const uint16_t*>(w_k); pr.Bm[1] = static_cast<const uint16_t*>(w_v);
+    pr.ldb[0] = pr.ldb[1] = ldw;
+    pr.K[0] = pr.K[1] = N; pr.nseg = 2;
+    pr.C = static_cast<uint16_t*>(dx); pr.ldc = lddx;
+    fill_grid(g, M, Dm, 1);
+    // B[k = n][col = dm]: W [Dm][N] has k contiguous, W [N][Dm] has the column contiguous
+    return static_cast<int>(launch_gemm(g, false, w_in_major == 0, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_t lddkv, void* dw_k, void* dw_v,
+              int64_t ldw, int32_t w_in_major, int32_t M, int32_t Dm, int32_t N, void* stream) {
+    LVX_TRY(check_gemm_ptr(x, ldx));
+    LVX_TRY(check_gemm_ptr(dk, lddkv));
+    LVX_TRY(check_gemm_ptr(dv, lddkv));
+    LVX_TRY(check_gemm_ptr(dw_k, ldw));
+    LVX_TRY(check_gemm_ptr(dw_v, ldw));
+    if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
+    if (ldx < Dm || lddkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
+    GemmParams g{};
+    const void* d[2] = {dk, dv};
+    void* c[2] = {dw_k, dw_v};
+    for (int i = 0; i < 2; ++i) {
+        GemmProblem& pr = g.prob[i];
+        if (w_in_major) {   // dW [Dm][N] = X^T dK
+            pr.A[0] = static_cast<const uint16_t*>(x); pr.lda[0] = ldx;
+            pr.Bm[0] = static_cast<const uint16_t*>(d[i]); pr.ldb[0] = lddkv;
+        } else {            // dW [N][Dm] = dK^T X
+            pr.A[0] = static_cast<const uint16_t*>(d[i]); pr.lda[0] = lddkv;
+            pr.Bm[0] = static_cast<const uint16_t*>(x); pr.ldb[0] = ldx;
+        }
+        pr.K[0] = M; pr.nseg = 1;
+        pr.C = static_cast<uint16_t*>(c[i]); pr.ldc = ldw;
+    }
+    if (w_in_major) fill_grid(g, Dm, N, 2);
+    else fill_grid(g, N, Dm, 2);
+    return static_cast<int>(launch_gemm(g, true, true, static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

@@ -1,0 +1,81 @@
+// Shared device helpers for the gfx950 (CDNA4) kernels: vector types, the
+// 32x32x16 bf16 MFMA wrapper with its operand/accumulator lane layout, bf16
+// packing, and the register-level 4x8 transpose used when a tile has to be
+// staged into LDS with its contraction index contiguous.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lvx {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int WAVE = 64;
+
+// D = A(32x16) * B(16x32) + C on one wavefront.  With lane l, g = l / 32:
+//   A operand: row i = l % 32, the 8 values are contraction slots (g, e), e = 0..7
+//   B operand: col j = l % 32, the 8 values are contraction slots (g, e)
+//   C/D      : col j = l % 32, register v holds row i = 8*(v/4) + 4*g + (v%4)
+// Slot (g, e) of A multiplies slot (g, e) of B; which logical k a slot stands
+// for is the caller's choice as long as both operands agree.
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Row of accumulator register v for lane-half g (see above).
+__device__ __forceinline__ int acc_row(int v, int g) { return 8 * (v >> 2) + 4 * g + (v & 3); }
+
+// When an accumulator tile is fed back as a B operand (its 32 rows become the
+// contraction index), registers 8*s .. 8*s+7 form k-step s and slot (g, e)
+// stands for row 16*s + 8*(e/4) + 4*g + (e%4).  The other operand is staged in
+// LDS with that row stored at column 16*s + 8*g + e, i.e. with bits 2 and 3 of
+// the row index exchanged:
+__device__ __forceinline__ int swap23(int r) {
+    return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 x = {lo, hi};
+    bf16x2 y = __builtin_convertvector(x, bf16x2);   // v_cvt_pk_bf16_f32, round-to-nearest-even
+    return __builtin_bit_cast(uint32_t, y);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 u) { return __builtin_bit_cast(bf16x8, u); }
+
+// 16-byte global load, zero when !ok.
+__device__ __forceinline__ u32x4 ldg16(const void* p, bool ok) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    return ok ? *reinterpret_cast<const u32x4*>(p) : z;
+}
+
+// r[i] = 8 bf16 of source row i (columns c..c+7), i = 0..3.
+// out[c] = the 4 values of column c (rows 0..3) packed as 4 bf16 = 8 bytes.
+__device__ __forceinline__ void transpose_4x8(const u32x4 r[4], u32x2 out[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t a = r[0][j], b = r[1][j], c = r[2][j], d = r[3][j];
+        out[2 * j][0] = (a & 0xffffu) | (b << 16);
+        out[2 * j][1] = (c & 0xffffu) | (d << 16);
+        out[2 * j + 1][0] = (a >> 16) | (b & 0xffff0000u);
+        out[2 * j + 1][1] = (c >> 16) | (d & 0xffff0000u);
+    }
+}
+
+// Work-groups are dealt to the 8 XCDs round-robin by linear id.  Remap so that
+// each XCD receives one contiguous range of the work list: neighbours in the
+// list (which share K/V or Q tiles) then share that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+    constexpr int NX = 8;
+    int per = (total + NX - 1) / NX;
+    return (bid % NX) * per + bid / NX;      // caller drops ids >= total
+}
+
+}  // namespace lvx

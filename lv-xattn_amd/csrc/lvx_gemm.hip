@@ -1,0 +1,156 @@
+// bf16 GEMM for the K/V recompute (K = X W_k, V = X W_v), its input gradient
+// (dX = dK W_k^T + dV W_v^T, one GEMM whose contraction runs over two operand
+// pairs) and the weight gradients (dW = X^T dK).  fp32 accumulate on
+// v_mfma_f32_32x32x16_bf16, bf16 output.
+//
+// A work-group computes a 128 x 128 tile of C with 4 waves (64 x 64 each, 2 x 2
+// MFMA tiles), stepping 64 along the contraction.  Both operand tiles are
+// staged in LDS with the contraction index contiguous ([128][64+8]); an operand
+// whose memory order has the other index contiguous is transposed in registers
+// on its way in.  The MFMA computes C^T (A operand = rows of the B tile), so a
+// lane ends up with 4 consecutive columns of one C row and stores 8 bytes.
+#include "lvx_common.hpp"
+#include "lvx_kernels.hpp"
+
+namespace lvx {
+
+namespace {
+
+constexpr int TM = 128, TN = 128, BK = 64;
+constexpr int LS = BK + 8;   // LDS row stride (elements)
+
+// Load the [128 rows][64 k] tile starting at (r0, k0) into 4 registers of 16 B.
+// CONTIG_K: memory is [row][k]; otherwise memory is [k][row].
+template <bool ROW_CONTIG>
+__device__ __forceinline__ void tile_load(u32x4 pre[4], const uint16_t* base, int64_t ld, int r0, int k0,
+                                          int R, int K, int tid) {
+    if (!ROW_CONTIG) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + 256 * i;
+            const int r = r0 + (c >> 3), k = k0 + (c & 7) * 8;
+            pre[i] = ldg16(base + (int64_t)r * ld + k, r < R && k < K);
+        }
+    } else {
+        const int rchunk = tid & 15, kgroup = tid >> 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + 4 * kgroup + i, r = r0 + 8 * rchunk;
+            pre[i] = ldg16(base + (int64_t)k * ld + r, k < K && r < R);
+        }
+    }
+}
+
+template <bool ROW_CONTIG>
+__device__ __forceinline__ void tile_store(const u32x4 pre[4], uint16_t* lds, int tid) {
+    if (!ROW_CONTIG) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + 256 * i;
+            *reinterpret_cast<u32x4*>(&lds[(c >> 3) * LS + (c & 7) * 8]) = pre[i];
+        }
+    } else {
+        const int rchunk = tid & 15, kgroup = tid >> 4;
+        u32x2 t8[8];
+        transpose_4x8(pre, t8);
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            *reinterpret_cast<u32x2*>(&lds[(8 * rchunk + r) * LS + 4 * kgroup]) = t8[r];
+    }
+}
+
+template <bool A_MCONTIG, bool B_NCONTIG>
+__global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[TM * LS];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[TN * LS];
+
+    const int wid = xcd_remap(blockIdx.x, p.total_wg);
+    if (wid >= p.total_wg) return;
+    const int tn = wid % p.tiles_n;
+    const int t1 = wid / p.tiles_n;
+    const int tm = t1 % p.tiles_m;
+    const GemmProblem& pr = p.prob[t1 / p.tiles_m];
+    const int m0 = tm * TM, n0 = tn * TN;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    f32x16 acc[2][2];   // [n tile][m tile]
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+    const int steps0 = (pr.K[0] + BK - 1) / BK;
+    const int steps1 = pr.nseg > 1 ? (pr.K[1] + BK - 1) / BK : 0;
+    const int steps = steps0 + steps1;
+
+    u32x4 apre[4], bpre[4];
+    auto prefetch = [&](int s) {
+        const int seg = s >= steps0 ? 1 : 0;
+        const int k0 = (seg ? s - steps0 : s) * BK;
+        tile_load<A_MCONTIG>(apre, pr.A[seg], pr.lda[seg], m0, k0, p.M, pr.K[seg], tid);
+        tile_load<B_NCONTIG>(bpre, pr.Bm[seg], pr.ldb[seg], n0, k0, p.N, pr.K[seg], tid);
+    };
+    if (steps > 0) prefetch(0);
+
+    for (int s = 0; s < steps; ++s) {
+        __syncthreads();
+        tile_store<A_MCONTIG>(apre, As, tid);
+        tile_store<B_NCONTIG>(bpre, Bs, tid);
+        __syncthreads();
+        if (s + 1 < steps) prefetch(s + 1);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            bf16x8 am[2], bn[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                am[t] = *reinterpret_cast<const bf16x8*>(&As[(64 * wm + 32 * t + l32) * LS + kk * 16 + g * 8]);
+                bn[t] = *reinterpret_cast<const bf16x8*>(&Bs[(64 * wn + 32 * t + l32) * LS + kk * 16 + g * 8]);
+            }
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt) acc[nt][mt] = mfma32(bn[nt], am[mt], acc[nt][mt]);
+        }
+    }
+
+    // C^T tile: accumulator rows = n, cols = m
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+        const int m = m0 + 64 * wm + 32 * mt + l32;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                const int n = n0 + 64 * wn + 32 * nt + 8 * vg + 4 * g;
+                if (n < p.N) {
+                    u32x2 w;
+                    w[0] = pack_bf16(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
+                    w[1] = pack_bf16(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
+                    *reinterpret_cast<u32x2*>(pr.C + (int64_t)m * pr.ldc + n) = w;
+                }
+            }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+    const int grid = ((p.total_wg + 7) / 8) * 8;
+    if (!a_mcontig && !b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<false, false>), dim3(grid), dim3(256), 0, st, p);
+    else if (!a_mcontig && b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<false, true>), dim3(grid), dim3(256), 0, st, p);
+    else if (a_mcontig && !b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<true, false>), dim3(grid), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL((gemm_kernel<true, true>), dim3(grid), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+}  // namespace lvx

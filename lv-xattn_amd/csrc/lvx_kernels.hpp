@@ -1,0 +1,111 @@
+// Internal launch interface between the C-ABI layer (lvx_api.hip) and the
+// kernel translation units.  All sizes have been validated by the caller.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lvx {
+
+struct Strides3 {
+    int64_t b, h, s;
+};
+
+struct FwdParams {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint16_t* o;
+    float* lse;
+    Strides3 qs, ks, vs, os;
+    int64_t o_split_stride;    // elements between the partial O of two key splits
+    int64_t lse_split_stride;  // floats between the partial LSE of two key splits
+    int64_t lse_bh_stride;     // floats between two (b, h) rows of LSE
+    const int32_t* kv_len;
+    const int32_t* kv_start;
+    const int32_t* kv_end;
+    int B, Hq, Hkv, Lq, Lkv;
+    int G;                     // q heads per kv head
+    int HG;                    // q heads a work-group covers (one per wave)
+    int RS;                    // 32-row sub-tiles a work-group covers per head
+    int row_begin, row_end;
+    int n_row_tiles, n_head_groups, nsplit, split_len, total_wg;
+    float scale, scale_log2e;
+};
+
+struct MergeParams {
+    uint16_t* o_acc;
+    float* l_acc;
+    const uint16_t* o_part;
+    const float* l_part;
+    Strides3 oa, op;
+    int64_t o_part_stride;     // elements between consecutive partials
+    int64_t l_part_stride;     // floats between consecutive partials
+    int64_t l_acc_bh, l_part_bh;
+    int nparts;
+    int use_acc;               // 1: fold into the existing accumulator, 0: overwrite
+    int B, Hq, Lq, row_begin, row_end;
+};
+
+struct PreParams {
+    const uint16_t* o;
+    const uint16_t* dout;
+    float* delta;
+    Strides3 os, ds;
+    int B, Hq, Lq, row_begin, row_end;
+};
+
+struct BwdParams {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    const uint16_t* dout;
+    const float* lse;
+    const float* delta;
+    float* dq_acc;
+    void* dk;
+    void* dv;
+    Strides3 qs, ks, vs, dos, dks, dvs;
+    const int32_t* kv_len;
+    const int32_t* kv_start;
+    const int32_t* kv_end;
+    int B, Hq, Hkv, Lq, Lkv, G;
+    int row_begin, row_end;
+    int n_kv_blocks, total_wg;
+    int dkv_accumulate;
+    float scale, scale_log2e;
+};
+
+struct CastParams {
+    const float* src;
+    uint16_t* dst;
+    Strides3 ds;
+    int B, H, L;
+};
+
+// One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].
+struct GemmProblem {
+    const uint16_t* A[2];
+    const uint16_t* Bm[2];
+    int64_t lda[2], ldb[2];
+    int K[2];
+    int nseg;
+    uint16_t* C;
+    int64_t ldc;
+};
+
+struct GemmParams {
+    GemmProblem prob[2];
+    int nprob;
+    int M, N;
+    int tiles_m, tiles_n, total_wg;
+};
+
+hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st);
+hipError_t launch_merge(const MergeParams& p, hipStream_t st);
+hipError_t launch_preprocess(const PreParams& p, hipStream_t st);
+hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);
+hipError_t launch_cast(const CastParams& p, hipStream_t st);
+// a_mcontig: A is stored [K][M] (m contiguous); b_ncontig: B is stored [K][N].
+hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st);
+
+}  // namespace lvx

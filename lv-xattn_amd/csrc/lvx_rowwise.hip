@@ -1,0 +1,156 @@
+// The HBM-bound row-wise kernels of the path: the LSE rescale-merge, the
+// backward preprocess (delta = rowsum(O * dO)) and the final fp32 -> bf16
+// rounding of an accumulator.  head_dim is 128: a row is 16 lanes x 16 bytes,
+// so a 256-thread group streams 16 rows per pass with fully coalesced 256-byte
+// row segments.
+#include "lvx_common.hpp"
+#include "lvx_kernels.hpp"
+
+namespace lvx {
+
+namespace {
+
+constexpr int D = 128;
+constexpr int MAX_PARTS = 16;
+
+__device__ __forceinline__ void unpack8(u32x4 u, float f[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f[2 * j] = bf16_lo(u[j]);
+        f[2 * j + 1] = bf16_hi(u[j]);
+    }
+}
+
+// (o_acc, l_acc) <- merge(acc?, part_0 .. part_{n-1}) for every (b, h, row).
+__global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
+    const int nrows = p.row_end - p.row_begin;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int chunk = (int)(idx & 15);
+    const int64_t r = idx >> 4;
+    if (r >= (int64_t)p.B * p.Hq * nrows) return;
+    const int row = p.row_begin + (int)(r % nrows);
+    const int bh = (int)(r / nrows);
+    const int b = bh / p.Hq, h = bh % p.Hq;
+
+    float la = -INFINITY;
+    if (p.use_acc) la = p.l_acc[(int64_t)bh * p.l_acc_bh + row];
+    float lp[MAX_PARTS];
+    float m = la;
+#pragma unroll
+    for (int i = 0; i < MAX_PARTS; ++i) {
+        if (i < p.nparts) {
+            lp[i] = p.l_part[i * p.l_part_stride + (int64_t)bh * p.l_part_bh + row];
+            m = fmaxf(m, lp[i]);
+        }
+    }
+    const float ms = (m == -INFINITY) ? 0.f : m;
+    float wa = __expf(la - ms);
+    float den = wa;
+#pragma unroll
+    for (int i = 0; i < MAX_PARTS; ++i) {
+        if (i < p.nparts) {
+            lp[i] = __expf(lp[i] - ms);
+            den += lp[i];
+        }
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+
+    float out[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = 0.f;
+    uint16_t* oa = p.o_acc + b * p.oa.b + h * p.oa.h + (int64_t)row * p.oa.s + chunk * 8;
+    if (p.use_acc) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(oa), f);
+        const float w = wa * inv;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = f[j] * w;
+    }
+    const uint16_t* op = p.o_part + b * p.op.b + h * p.op.h + (int64_t)row * p.op.s + chunk * 8;
+#pragma unroll
+    for (int i = 0; i < MAX_PARTS; ++i) {
+        if (i < p.nparts) {
+            float f[8];
+            unpack8(*reinterpret_cast<const u32x4*>(op + i * p.o_part_stride), f);
+            const float w = lp[i] * inv;
+            // a part with weight 0 may hold anything (it saw no key)
+            if (w > 0.f) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) out[j] = fmaf(f[j], w, out[j]);
+            }
+        }
+    }
+    u32x4 u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u[j] = pack_bf16(out[2 * j], out[2 * j + 1]);
+    *reinterpret_cast<u32x4*>(oa) = u;
+    if (chunk == 0) p.l_acc[(int64_t)bh * p.l_acc_bh + row] = den > 0.f ? ms + __logf(den) : -INFINITY;
+}
+
+__global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
+    const int nrows = p.row_end - p.row_begin;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int chunk = (int)(idx & 15);
+    const int64_t r = idx >> 4;
+    const bool ok = r < (int64_t)p.B * p.Hq * nrows;   // whole 16-lane groups share `ok`
+    const int64_t rr = ok ? r : 0;
+    const int row = p.row_begin + (int)(rr % nrows);
+    const int bh = (int)(rr / nrows);
+    const int b = bh / p.Hq, h = bh % p.Hq;
+    float fo[8], fd[8];
+    unpack8(ldg16(p.o + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s + chunk * 8, ok), fo);
+    unpack8(ldg16(p.dout + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8, ok), fd);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
+    s += __shfl_xor(s, 8);
+    s += __shfl_xor(s, 4);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 1);
+    if (ok && chunk == 0) p.delta[(int64_t)bh * p.Lq + row] = s;
+}
+
+__global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int chunk = (int)(idx & 15);
+    const int64_t r = idx >> 4;
+    if (r >= (int64_t)p.B * p.H * p.L) return;
+    const int row = (int)(r % p.L);
+    const int bh = (int)(r / p.L);
+    const int b = bh / p.H, h = bh % p.H;
+    const f32x4* s = reinterpret_cast<const f32x4*>(p.src + r * D + chunk * 8);
+    const f32x4 a = s[0], c = s[1];
+    u32x4 u;
+    u[0] = pack_bf16(a[0], a[1]);
+    u[1] = pack_bf16(a[2], a[3]);
+    u[2] = pack_bf16(c[0], c[1]);
+    u[3] = pack_bf16(c[2], c[3]);
+    *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
+}
+
+inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
+
+}  // namespace
+
+hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(merge_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(preprocess_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_cast(const CastParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.B * p.H * p.L;
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(cast_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+}  // namespace lvx

@@ -1,0 +1,150 @@
+"""Host round loops of the cross-attention hot path, with the call signatures
+of the reference's `_attn_forward` / `_attn_backward`
+(lv_xattn/attn.py:297-298 and :437 there).
+
+The reference moves each query block round a ring of P GPUs; every GPU
+computes that block's partial result against its own stationary K/V shard and
+folds it into the (O, LSE) accumulator travelling with the block.  On one
+MI355X the P visits are P rounds over the query blocks of `q`, all against the
+one local shard: round r computes block r's partial with `lvx_fwd`, then
+`lvx_merge` folds it into that block's accumulator (what would have arrived
+from the left neighbour: `acc_in`, default the identity (0, -inf)).
+
+Everything runs on the current PyTorch stream; nothing here synchronises.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import ops
+from .async_communication import get_sequence_parallel_size, workspace
+from .ops import Mask
+
+__all__ = ["_attn_forward", "_attn_backward", "q_block_bounds", "Mask"]
+
+
+def q_block_bounds(lq: int, rounds: int) -> List[Tuple[int, int]]:
+    """Row window of each of the P query blocks: ceil(Lq/P) rows, the tail
+    shorter (the reference needs Lq % P == 0: test.py:160)."""
+    lb = -(-lq // rounds)
+    return [(min(r * lb, lq), min((r + 1) * lb, lq)) for r in range(rounds)]
+
+
+def _usable(t: torch.Tensor) -> torch.Tensor:
+    """The kernels take any [B,H,S,D] view with unit last stride and the other
+    strides multiples of 8 elements; anything else is copied once."""
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        return t.contiguous()
+    return t
+
+
+def _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args):
+    if causal:
+        # the reference applies the triangle to rank-local indices only
+        # (lv_xattn/attn.py:229,237), which means nothing once blocks travel
+        raise ValueError("causal=True is not defined for cross-attention over travelling query blocks")
+    if bias_func is not None or len(local_bias_args) or len(remote_bias_args):
+        raise NotImplementedError(
+            "dense additive bias_func is not implemented on the gfx950 path; "
+            "pass the compact interval form via mask=Mask(kv_len, kv_start, kv_end)")
+
+
+def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
+                  local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
+                  rounds: Optional[int] = None, mask: Optional[Mask] = None,
+                  acc_in: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                  kv_splits: int = 1, batched: bool = False):
+    """Returns (q, k, v, o, L) like the reference (attn.py:435): o [B,Hq,Lq,D]
+    bf16, L [B*Hq, Lq] fp32 natural-log LSE of sm_scale * q k^T.
+
+    q [B,Hq,Lq,D] holds all P query blocks back to back; k, v [B,Hkv,Lkv,D] are
+    the local shard at Hkv heads (Hkv | Hq; expanded in-kernel).
+    `comm_mode` and `no_overlap` are accepted and ignored (no transport).
+    Keyword-only additions: `rounds` (P; default the size set by
+    initialize_distributed), `mask`, `acc_in` = (O_in bf16 [B,Hq,Lq,D],
+    L_in fp32 [B*Hq,Lq]) for every block, `kv_splits` (key ranges per round
+    computed by separate work-groups), `batched` (one launch over all P blocks
+    instead of one per round)."""
+    _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
+    q_, k_, v_ = _usable(q), _usable(k), _usable(v)
+    B, Hq, Lq, D = q_.shape
+    P = rounds if rounds is not None else get_sequence_parallel_size()
+    dev = q_.device
+    if mask is not None:
+        mask = mask.to(dev)
+
+    if acc_in is None:
+        o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
+        L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
+    else:
+        o = acc_in[0].to(dtype=q_.dtype).clone(memory_format=torch.contiguous_format)
+        L = acc_in[1].to(torch.float32).reshape(B * Hq, Lq).clone()
+
+    windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
+    max_rows = max(r1 - r0 for r0, r1 in windows)
+    ws = None
+    if kv_splits > 1:
+        nbytes = ops.fwd_workspace_bytes(q_, k_, max_rows, kv_splits)
+        ws = workspace("fwd_split", (nbytes,), torch.uint8, dev)
+
+    if acc_in is None:
+        # merging into the identity returns the partial itself: write in place
+        for r0, r1 in windows:
+            ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws)
+    else:
+        o_part = workspace("fwd_o_part", (B, Hq, Lq, D), q_.dtype, dev)
+        l_part = workspace("fwd_l_part", (B * Hq, Lq), torch.float32, dev)
+        for r0, r1 in windows:
+            ops.fwd(q_, k_, v_, o_part, l_part, sm_scale, r0, r1 - r0, mask, kv_splits, ws)
+            ops.merge(o, L, o_part, l_part, r0, r1 - r0)
+    return q, k, v, o, L
+
+
+def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engine,
+                   bias_func=None, local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
+                   rounds: Optional[int] = None, mask: Optional[Mask] = None, batched: bool = False):
+    """Returns (dq, dk, dv) like the reference (attn.py:545): dq [B,Hq,Lq,D];
+    dk, dv [B,Hkv,Lkv,D]-shaped views of [B,Lkv,Hkv,D] memory, at the Hkv heads
+    k and v came in with.  `o` and `L` are the finally merged forward results;
+    every round uses them, so per-round contributions simply add
+    (attn.py:465-468, 509-527).  dQ, dK, dV are summed in fp32 across q heads of
+    a group and across rounds and rounded to bf16 once.
+    `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored."""
+    _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
+    q_, k_, v_, o_, do_ = (_usable(t) for t in (q, k, v, o, do))
+    B, Hq, Lq, D = q_.shape
+    Hkv, Lkv = k_.shape[1], k_.shape[2]
+    P = rounds if rounds is not None else get_sequence_parallel_size()
+    dev = q_.device
+    if mask is not None:
+        mask = mask.to(dev)
+    L_ = L.to(torch.float32).reshape(B * Hq, Lq).contiguous()
+
+    delta = workspace("bwd_delta", (B * Hq, Lq), torch.float32, dev)
+    dq_acc = workspace("bwd_dq_acc", (B, Hq, Lq, D), torch.float32, dev)
+    dq_acc.zero_()
+    dq = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
+    dk = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
+    dv = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
+
+    windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
+    if len(windows) == 1:
+        r0, r1 = windows[0]
+        ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
+        ops.bwd(q_, k_, v_, do_, L_, delta, dq_acc, dk, dv, sm_scale, r0, r1 - r0, mask, accumulate_dkv=False)
+    else:
+        dk_acc = workspace("bwd_dk_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
+        dv_acc = workspace("bwd_dv_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
+        dk_acc.zero_()
+        dv_acc.zero_()
+        for r0, r1 in windows:
+            ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
+            ops.bwd(q_, k_, v_, do_, L_, delta, dq_acc, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
+                    accumulate_dkv=True)
+        # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
+        ops.cast_f32_bf16(dk_acc.transpose(1, 2), dk.transpose(1, 2))
+        ops.cast_f32_bf16(dv_acc.transpose(1, 2), dv.transpose(1, 2))
+    ops.cast_f32_bf16(dq_acc, dq)
+    return dq, dk, dv

@@ -1,0 +1,100 @@
+"""The two autograd wrappers the reference's harnesses build around
+`_attn_forward` / `_attn_backward`:
+
+* `create_attention_class_save_qkv` - classic save-(q,k,v,o,L) function
+  (test.py:38-77 and test_llama3.py:125-178 there);
+* `create_attention_class`          - the K/V-RECOMPUTE variant
+  (test_llama3.py:180-245): forward keeps only (x, o, L); backward re-runs the
+  projection of the shared visual hidden states instead of loading stored K/V.
+
+Unlike the reference's recompute wrapper, which returns no gradients at all
+(test_llama3.py:243), backward here returns real ones, including the gradient
+that flows into the visual hidden states (dX_vis) and the projection weights.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+
+from . import ops
+from .attn import Mask, _attn_backward, _attn_forward
+from .async_communication import reset_global_memory_buffer
+
+
+def create_attention_class_save_qkv(attention_mode: str = "lv_xattn", no_overlap: bool = False,
+                                    rounds: Optional[int] = None, batched: bool = False):
+    """apply(q, k, v, causal, sm_scale, bias_func=None, local_bias_args=[],
+    remote_bias_args=[], mask=None) -> o"""
+    if attention_mode != "lv_xattn":
+        raise ValueError("only attention_mode='lv_xattn' exists on this path")
+
+    class _attention(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, q, k, v, causal, sm_scale, bias_func=None, local_bias_args=[],
+                    remote_bias_args=[], mask=None):
+            q, k, v, o, L = _attn_forward(q, k, v, causal, sm_scale, None, bias_func, local_bias_args,
+                                          remote_bias_args, no_overlap, rounds=rounds, mask=mask,
+                                          batched=batched)
+            ctx.save_for_backward(q, k, v, o, L)
+            ctx.sm_scale, ctx.causal, ctx.mask = sm_scale, causal, mask
+            return o
+
+        @staticmethod
+        def backward(ctx, do):
+            q, k, v, o, L = ctx.saved_tensors
+            dq, dk, dv = _attn_backward(do, q, k, v, o, L, ctx.causal, ctx.sm_scale, None, "flash",
+                                        no_overlap=no_overlap, rounds=rounds, mask=ctx.mask, batched=batched)
+            return dq, dk, dv, None, None, None, None, None, None
+
+    return _attention
+
+
+class KVProjection:
+    """The K/V half of the reference's `project` closure
+    (test_llama3.py:395-398): K = X_vis W_k, V = X_vis W_v, computed by the
+    gfx950 GEMM and handed to attention in [B, Lkv, Hkv, D] memory order."""
+
+    def __init__(self, w_k: torch.Tensor, w_v: torch.Tensor, n_kv_heads: int, w_in_major: bool = True):
+        self.w_k, self.w_v, self.n_kv_heads, self.w_in_major = w_k, w_v, n_kv_heads, w_in_major
+
+    def __call__(self, x_vis: torch.Tensor):
+        return ops.kv_proj(x_vis, self.w_k, self.w_v, self.n_kv_heads, self.w_in_major)
+
+
+def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = False,
+                           rounds: Optional[int] = None, batched: bool = False,
+                           weight_grads: bool = False):
+    """apply(q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None) -> o
+
+    Forward: K, V = kv_proj(x_vis); o, L = attention; saves (q, x_vis, w_k, w_v,
+    o, L) - K and V are dropped.  Backward: recomputes K, V by the same GEMMs,
+    runs the attention backward, then dX_vis = dK W_k^T + dV W_v^T (and, with
+    `weight_grads`, dW_k = X^T dK, dW_v = X^T dV)."""
+    if attention_mode != "lv_xattn":
+        raise ValueError("only attention_mode='lv_xattn' exists on this path")
+
+    class _attention(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None):
+            k, v = ops.kv_proj(x_vis, w_k, w_v, n_kv_heads)
+            _, _, _, o, L = _attn_forward(q, k, v, False, sm_scale, None, no_overlap=no_overlap,
+                                          rounds=rounds, mask=mask, batched=batched)
+            ctx.save_for_backward(q, x_vis, w_k, w_v, o, L)
+            ctx.n_kv_heads, ctx.sm_scale, ctx.mask = n_kv_heads, sm_scale, mask
+            reset_global_memory_buffer(attention_mode)
+            return o
+
+        @staticmethod
+        def backward(ctx, do):
+            q, x_vis, w_k, w_v, o, L = ctx.saved_tensors
+            k, v = ops.kv_proj(x_vis, w_k, w_v, ctx.n_kv_heads)          # recompute
+            dq, dk, dv = _attn_backward(do, q, k, v, o, L, False, ctx.sm_scale, None, "flash",
+                                        no_overlap=no_overlap, rounds=rounds, mask=ctx.mask, batched=batched)
+            dx = ops.dx_vis(dk, dv, w_k, w_v)
+            dwk = dwv = None
+            if weight_grads:
+                dwk, dwv = ops.dw_kv(x_vis, dk, dv)
+            return dq, dx, dwk, dwv, None, None, None
+
+    return _attention

@@ -1,0 +1,200 @@
+"""One Python function per C entry point of liblvx.so, taking torch tensors.
+
+These are the device operators the round loops in ``attn.py`` are made of; each
+queues its kernel(s) on the current PyTorch stream and returns immediately.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import AttnShape, LvxError, check, load, ptr, stream_ptr, t4
+
+
+@dataclass
+class Mask:
+    """Compact mask of a ragged / Llama-3.2-style batch.
+
+    kv_len   int32 [B]      valid visual tokens per sample (None: all)
+    kv_start int32 [B, Lq]  first visible visual token of each text row
+    kv_end   int32 [B, Lq]  one past the last visible token (None: no interval mask)
+    A row whose interval is empty sees nothing: O = 0, LSE = -inf, dQ = 0.
+    """
+    kv_len: Optional[torch.Tensor] = None
+    kv_start: Optional[torch.Tensor] = None
+    kv_end: Optional[torch.Tensor] = None
+
+    def to(self, device) -> "Mask":
+        f = lambda t: None if t is None else t.to(device=device, dtype=torch.int32).contiguous()
+        return Mask(f(self.kv_len), f(self.kv_start), f(self.kv_end))
+
+
+def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask]) -> AttnShape:
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16:
+        raise LvxError(f"bf16 tensors required, got {q.dtype} / {k.dtype}")
+    B, Hq, Lq, D = q.shape
+    Bk, Hkv, Lkv, Dk = k.shape
+    if B != Bk or D != Dk:
+        raise LvxError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
+    s = AttnShape(B, Hq, Hkv, D, Lq, Lkv, _lib.LVX_BF16, float(scale), None, None, None)
+    if mask is not None:
+        for name in ("kv_len", "kv_start", "kv_end"):
+            t = getattr(mask, name)
+            if t is None:
+                continue
+            want = (B,) if name == "kv_len" else (B, Lq)
+            if t.dtype != torch.int32 or tuple(t.shape) != want or not t.is_contiguous() or t.device != q.device:
+                raise LvxError(f"mask.{name} must be a contiguous int32 {want} tensor on {q.device}")
+            setattr(s, name, t.data_ptr())
+    return s
+
+
+def fwd_workspace_bytes(q, k, row_count: int, kv_splits: int) -> int:
+    s = _shape(q, k, 1.0, None)
+    return int(load().lvx_fwd_workspace_bytes(C.byref(s), row_count, kv_splits))
+
+
+def fwd(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask] = None,
+        kv_splits: int = 1, workspace: Optional[torch.Tensor] = None) -> None:
+    """Partial O (bf16) and LSE (fp32 [B*Hq, Lq]) of text rows
+    [row_begin, row_begin+row_count) against the whole local K/V shard."""
+    s = _shape(q, k, scale, mask)
+    if row_count is None:
+        row_count = q.shape[2] - row_begin
+    _check_lse(lse, q)
+    ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    rc = load().lvx_fwd(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(o)),
+                        lse.data_ptr(), row_begin, row_count, kv_splits, ws_ptr, ws_bytes, stream_ptr())
+    check(rc, "lvx_fwd")
+
+
+def merge(o_acc, l_acc, o_part, l_part, row_begin=0, row_count=None) -> None:
+    """(o_acc, l_acc) <- LSE-merge of itself with (o_part, l_part), in place."""
+    B, Hq, Lq, D = o_acc.shape
+    s = AttnShape(B, Hq, Hq, D, Lq, 1, _lib.LVX_BF16, 1.0, None, None, None)
+    if row_count is None:
+        row_count = Lq - row_begin
+    _check_lse(l_acc, o_acc)
+    _check_lse(l_part, o_acc)
+    rc = load().lvx_merge(C.byref(s), C.byref(t4(o_acc)), l_acc.data_ptr(), C.byref(t4(o_part)),
+                          l_part.data_ptr(), row_begin, row_count, stream_ptr())
+    check(rc, "lvx_merge")
+
+
+def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
+    B, Hq, Lq, D = o.shape
+    s = AttnShape(B, Hq, Hq, D, Lq, 1, _lib.LVX_BF16, 1.0, None, None, None)
+    if row_count is None:
+        row_count = Lq - row_begin
+    _check_lse(delta, o)
+    rc = load().lvx_bwd_preprocess(C.byref(s), C.byref(t4(o)), C.byref(t4(dout)), delta.data_ptr(),
+                                   row_begin, row_count, stream_ptr())
+    check(rc, "lvx_bwd_preprocess")
+
+
+def bwd(q, k, v, dout, lse, delta, dq_acc, dk, dv, scale, row_begin=0, row_count=None,
+        mask: Optional[Mask] = None, accumulate_dkv: bool = False) -> None:
+    """Adds the selected rows' contribution to dq_acc (fp32 [B,Hq,Lq,D]) and
+    writes (bf16) or accumulates (fp32) dk, dv at Hkv heads."""
+    s = _shape(q, k, scale, mask)
+    if row_count is None:
+        row_count = q.shape[2] - row_begin
+    _check_lse(lse, q)
+    _check_lse(delta, q)
+    if dq_acc.dtype != torch.float32 or not dq_acc.is_contiguous() or dq_acc.shape != q.shape:
+        raise LvxError("dq_acc must be a contiguous fp32 tensor shaped like q")
+    want = torch.float32 if accumulate_dkv else torch.bfloat16
+    if dk.dtype != want or dv.dtype != want or dk.shape != k.shape or dv.shape != k.shape:
+        raise LvxError(f"dk/dv must be {want} tensors shaped like k")
+    rc = load().lvx_bwd(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(dout)),
+                        lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr(), C.byref(t4(dk)), C.byref(t4(dv)),
+                        1 if accumulate_dkv else 0, row_begin, row_count, stream_ptr())
+    check(rc, "lvx_bwd")
+
+
+def cast_f32_bf16(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst (bf16, [B,H,L,D] any strides) = src (fp32, memory order [B,H,L,D])."""
+    B, H, L, D = dst.shape
+    if src.dtype != torch.float32 or src.numel() != dst.numel() or dst.dtype != torch.bfloat16:
+        raise LvxError("cast_f32_bf16: fp32 source and bf16 destination of equal size required")
+    rc = load().lvx_cast_f32_bf16(src.data_ptr(), C.byref(t4(dst)), B, H, L, D, stream_ptr())
+    check(rc, "lvx_cast_f32_bf16")
+
+
+def _rows2d(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
+    """[..., C] tensor whose leading dims collapse to rows with one stride."""
+    if t.dtype != torch.bfloat16:
+        raise LvxError(f"{name}: bf16 required")
+    t2 = t.reshape(-1, t.shape[-1]) if t.is_contiguous() else None
+    if t2 is None:
+        raise LvxError(f"{name}: contiguous tensor required")
+    return t2.data_ptr(), t2.shape[0], t2.stride(0)
+
+
+def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True):
+    """K, V = X W_k, X W_v.  x_vis [B, Lkv, Dm]; W [Dm, Hkv*D] (w_in_major) or
+    [Hkv*D, Dm] (torch.nn.Linear.weight).  Returns [B, Hkv, Lkv, D] views of
+    [B, Lkv, Hkv, D] memory."""
+    B, Lkv, Dm = x_vis.shape
+    N = w_k.shape[1] if w_in_major else w_k.shape[0]
+    xp, M, ldx = _rows2d(x_vis, "x_vis")
+    wkp, _, ldw = _rows2d(w_k, "w_k")
+    wvp, _, ldw2 = _rows2d(w_v, "w_v")
+    if ldw != ldw2 or w_k.shape != w_v.shape:
+        raise LvxError("w_k and w_v must have the same shape")
+    k = torch.empty(B, Lkv, N, dtype=torch.bfloat16, device=x_vis.device)
+    v = torch.empty_like(k)
+    rc = load().lvx_kv_proj(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
+                            M, Dm, N, stream_ptr())
+    check(rc, "lvx_kv_proj")
+    D = N // n_kv_heads
+    return (k.view(B, Lkv, n_kv_heads, D).transpose(1, 2), v.view(B, Lkv, n_kv_heads, D).transpose(1, 2))
+
+
+def _token_major(t: torch.Tensor, name: str) -> torch.Tensor:
+    """[B, Hkv, Lkv, D] view whose memory is [B, Lkv, Hkv, D] -> [B*Lkv, Hkv*D]."""
+    tm = t.transpose(1, 2)
+    if not tm.is_contiguous():
+        raise LvxError(f"{name} must be a [B,Hkv,Lkv,D] view of contiguous [B,Lkv,Hkv,D] memory")
+    return tm.reshape(tm.shape[0] * tm.shape[1], -1)
+
+
+def dx_vis(dk, dv, w_k, w_v, w_in_major: bool = True) -> torch.Tensor:
+    """dX = dK W_k^T + dV W_v^T -> [B, Lkv, Dm]."""
+    B, Hkv, Lkv, D = dk.shape
+    dk2, dv2 = _token_major(dk, "dk"), _token_major(dv, "dv")
+    N = Hkv * D
+    Dm = w_k.shape[0] if w_in_major else w_k.shape[1]
+    wkp, _, ldw = _rows2d(w_k, "w_k")
+    wvp, _, _ = _rows2d(w_v, "w_v")
+    dx = torch.empty(B, Lkv, Dm, dtype=torch.bfloat16, device=dk.device)
+    rc = load().lvx_dx_vis(dk2.data_ptr(), dv2.data_ptr(), N, wkp, wvp, ldw, 1 if w_in_major else 0,
+                           dx.data_ptr(), Dm, B * Lkv, Dm, N, stream_ptr())
+    check(rc, "lvx_dx_vis")
+    return dx
+
+
+def dw_kv(x_vis, dk, dv, w_in_major: bool = True):
+    """dW_k = X^T dK, dW_v = X^T dV in the layout of W."""
+    B, Lkv, Dm = x_vis.shape
+    Hkv, D = dk.shape[1], dk.shape[3]
+    N = Hkv * D
+    dk2, dv2 = _token_major(dk, "dk"), _token_major(dv, "dv")
+    xp, M, ldx = _rows2d(x_vis, "x_vis")
+    shape = (Dm, N) if w_in_major else (N, Dm)
+    dwk = torch.empty(*shape, dtype=torch.bfloat16, device=x_vis.device)
+    dwv = torch.empty_like(dwk)
+    rc = load().lvx_dw_kv(xp, ldx, dk2.data_ptr(), dv2.data_ptr(), N, dwk.data_ptr(), dwv.data_ptr(), shape[1],
+                          1 if w_in_major else 0, M, Dm, N, stream_ptr())
+    check(rc, "lvx_dw_kv")
+    return dwk, dwv
+
+
+def _check_lse(l: torch.Tensor, q: torch.Tensor) -> None:
+    B, Hq, Lq, _ = q.shape
+    if l.dtype != torch.float32 or not l.is_contiguous() or l.numel() != B * Hq * Lq:
+        raise LvxError(f"LSE/delta must be contiguous fp32 with {B * Hq * Lq} elements ([B*Hq, Lq])")

@@ -1,0 +1,111 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every
+symbol the header declares, and rejects bad arguments on the host before any
+launch (so these calls are safe without a GPU)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lvx.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from lv_xattn import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("lvx_build", os.path.join(ROOT, "lv-xattn_amd", "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build(force=False)
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lvx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from lv_xattn import _lib
+    names = declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in lvx.h but not exported by liblvx.so"
+    assert sorted(_lib.SYMBOLS) == names, "ctypes table and header disagree"
+
+
+def test_version_and_error_strings(lib):
+    assert lib.lvx_version() == 100
+    assert lib.lvx_strerror(0) == b"ok"
+    for code in range(-8, 0):
+        assert lib.lvx_strerror(code) not in (b"", b"unknown lvx error")
+
+
+def _shape(**kw):
+    from lv_xattn._lib import AttnShape
+    d = dict(B=1, Hq=8, Hkv=2, D=128, Lq=64, Lkv=256, dtype=1, scale=0.1, kv_len=None, kv_start=None, kv_end=None)
+    d.update(kw)
+    return AttnShape(**d)
+
+
+def _t(ptr=0x1000, sb=8 * 64 * 128, sh=64 * 128, ss=128):
+    from lv_xattn._lib import Tensor4
+    return Tensor4(ptr, sb, sh, ss)
+
+
+def _fwd(lib, shape, q=None, k=None, v=None, o=None, lse=0x2000, rb=0, rc=64, splits=1, ws=None, wsb=0):
+    q, k, v, o = (x if x is not None else _t() for x in (q, k, v, o))
+    return lib.lvx_fwd(C.byref(shape), C.byref(q), C.byref(k), C.byref(v), C.byref(o), lse, rb, rc, splits, ws, wsb, None)
+
+
+def test_forward_rejects_bad_arguments_before_launch(lib):
+    assert _fwd(lib, _shape(D=64)) == -4
+    assert _fwd(lib, _shape(dtype=2)) == -5
+    assert _fwd(lib, _shape(Hq=7)) == -3
+    assert _fwd(lib, _shape(scale=0.0)) == -6
+    assert _fwd(lib, _shape(scale=float("nan"))) == -6
+    assert _fwd(lib, _shape(), q=_t(ptr=0)) == -1
+    assert _fwd(lib, _shape(), k=_t(ptr=0x1004)) == -2
+    assert _fwd(lib, _shape(), v=_t(ss=132)) == -2
+    assert _fwd(lib, _shape(), lse=None) == -1
+    assert _fwd(lib, _shape(), rb=32, rc=64) == -3
+    assert _fwd(lib, _shape(), splits=0) == -3
+    assert _fwd(lib, _shape(), splits=4) == -7            # no workspace given
+    assert _fwd(lib, _shape(kv_start=0x3000)) == -1       # kv_start without kv_end
+    assert _fwd(lib, _shape(), rc=0) == 0                 # empty window: nothing to do
+    assert lib.lvx_fwd(None, None, None, None, None, None, 0, 0, 1, None, 0, None) == -1
+
+
+def test_workspace_size(lib):
+    s = _shape()
+    assert lib.lvx_fwd_workspace_bytes(C.byref(s), 64, 1) == 0
+    assert lib.lvx_fwd_workspace_bytes(C.byref(s), 64, 4) == 4 * 8 * 64 * (128 * 2 + 4)
+
+
+def test_other_entry_points_reject_bad_arguments(lib):
+    s = _shape()
+    t = _t()
+    assert lib.lvx_merge(C.byref(s), C.byref(t), None, C.byref(t), 0x2000, 0, 64, None) == -1
+    assert lib.lvx_merge(C.byref(s), C.byref(t), 0x2000, C.byref(t), 0x2000, 0, 65, None) == -3
+    assert lib.lvx_bwd_preprocess(C.byref(s), C.byref(t), C.byref(_t(ptr=8)), 0x2000, 0, 64, None) == -2
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, None,
+                       C.byref(t), C.byref(t), 0, 0, 64, None) == -1
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, 0x3000,
+                       C.byref(t), C.byref(t), 2, 0, 64, None) == -3
+    assert lib.lvx_cast_f32_bf16(0x1000, C.byref(t), 1, 8, 64, 64, None) == -4
+    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, None) == -3
+    assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, None) == -1
+    assert lib.lvx_dx_vis(0x1000, 0x1100, 256, 0x2000, 0x3000, 250, 1, 0x4000, 512, 100, 512, 256, None) == -2
+    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, 0x3000, 128, 1, 100, 512, 256, None) == -3
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from lv_xattn import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liblvx.so")
+    with pytest.raises(_lib.LvxError, match="no CPU fallback"):
+        _lib.load()

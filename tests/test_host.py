@@ -1,0 +1,71 @@
+"""Host-side logic that needs no GPU: block bounds, the transport shims, the
+argument checks of the Python mirror of the reference API."""
+import pytest
+import torch
+
+import lv_xattn
+from lv_xattn import attn, ops
+from lv_xattn import async_communication as ac
+from oracle import lvx_oracle as orc
+
+
+def test_public_names_match_reference_package():
+    for name in ("_attn_forward", "_attn_backward", "initialize_distributed",
+                 "reset_global_memory_buffer", "get_sequence_parallel_group"):
+        assert hasattr(lv_xattn, name)
+
+
+def test_block_bounds_agree_with_oracle():
+    for lq, p in ((4096, 16), (3000, 16), (1777, 16), (10, 4), (5, 8)):
+        assert attn.q_block_bounds(lq, p) == orc.q_block_bounds(lq, p)
+        b = attn.q_block_bounds(lq, p)
+        assert b[0][0] == 0 and b[-1][1] == lq
+        assert all(b[i][1] == b[i + 1][0] for i in range(p - 1))
+
+
+def test_round_group_shim(monkeypatch):
+    monkeypatch.delenv("LVX_ROUNDS", raising=False)
+    monkeypatch.setenv("WORLD_SIZE", "16")
+    ac.initialize_distributed()
+    g = lv_xattn.get_sequence_parallel_group()
+    assert g.size() == 16 and g.rank() == 0
+    ac.initialize_distributed(4)
+    assert lv_xattn.get_sequence_parallel_group().size() == 4
+    with pytest.raises(ValueError):
+        ac.initialize_distributed(0)
+    ac.initialize_distributed(1)
+
+
+def test_workspace_cache_and_reset():
+    a = ac.workspace("t", (4, 4), torch.float32, "cpu")
+    assert ac.workspace("t", (4, 4), torch.float32, "cpu") is a
+    lv_xattn.reset_global_memory_buffer()
+    assert ac.workspace("t", (4, 4), torch.float32, "cpu") is not a
+    lv_xattn.reset_global_memory_buffer("lv_xattn")      # the reference passes the mode
+
+
+def test_causal_and_bias_are_rejected_explicitly():
+    q = torch.zeros(1, 4, 8, 128, dtype=torch.bfloat16)
+    k = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="causal"):
+        lv_xattn._attn_forward(q, k, k, True, 0.1, None)
+    with pytest.raises(NotImplementedError, match="bias_func"):
+        lv_xattn._attn_forward(q, k, k, False, 0.1, None, bias_func=lambda: None)
+    with pytest.raises(ValueError, match="causal"):
+        lv_xattn._attn_backward(q, q, k, k, q, torch.zeros(4, 8), True, 0.1, None, "flash")
+
+
+def test_shape_and_dtype_checks_raise_before_any_device_call():
+    q = torch.zeros(1, 4, 8, 128, dtype=torch.float16)
+    k = torch.zeros(1, 2, 8, 128, dtype=torch.float16)
+    with pytest.raises(ops.LvxError, match="bf16"):
+        ops._shape(q, k, 0.1, None)
+    qb, kb = q.bfloat16(), torch.zeros(2, 2, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(ops.LvxError, match="disagree"):
+        ops._shape(qb, kb, 0.1, None)
+    kb = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16)
+    bad = ops.Mask(kv_len=torch.zeros(3, dtype=torch.int32))
+    with pytest.raises(ops.LvxError, match="kv_len"):
+        ops._shape(qb, kb, 0.1, bad)
+    with pytest.raises(ops.LvxError, match="unit last stride"):
+        ops.t4(torch.zeros(1, 2, 128, 8, dtype=torch.bfloat16).transpose(2, 3))
