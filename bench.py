@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-GPU cross-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--mode batched|rounds]
+
+A step is one cross-attention layer, forward + backward with K/V recompute, at
+the Llama-3.2-11B-Vision shape of one GPU's share of a 16-way split (cfg2):
+K/V projection, P-round flash forward + LSE merge, K/V re-projection,
+backward preprocess, backward (dQ, dK, dV), dX_vis.  Inputs are synthetic,
+seeded, and resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "lv-xattn_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def flops(w, n_pairs):
+    f_fwd = 4.0 * w.D * w.Hq * n_pairs
+    f_bwd = 10.0 * w.D * w.Hq * n_pairs
+    f_proj = 4.0 * w.B * w.Lkv * w.Dm * w.Hkv * w.D if w.Dm else 0.0
+    return dict(fwd=f_fwd, bwd=f_bwd, proj=f_proj)
+
+
+class Layer:
+    """Device-side state of one benchmark layer and its step function."""
+
+    def __init__(self, w, mode, dev):
+        import torch
+        import lv_xattn
+        from lv_xattn import ops
+        self.torch, self.ops, self.lvx = torch, ops, lv_xattn
+        self.w, self.mode = w, mode
+        t = w.tensors
+        self.q = t["q"].to(dev)
+        self.do = t["do"].to(dev)
+        self.has_proj = w.Dm > 0
+        if self.has_proj:
+            self.x, self.wk, self.wv = t["x_vis"].to(dev), t["w_k"].to(dev), t["w_v"].to(dev)
+        else:
+            self.k, self.v = t["k"].to(dev), t["v"].to(dev)
+        self.mask = None
+        if w.kv_len is not None or "kv_start" in t:
+            kv_len = torch.tensor(w.kv_len, dtype=torch.int32) if w.kv_len else None
+            self.mask = lv_xattn.Mask(kv_len, t.get("kv_start"), t.get("kv_end")).to(dev)
+        B, Hq, Lq, D = self.q.shape
+        self.o_in = torch.zeros(B, Hq, Lq, D, dtype=torch.bfloat16, device=dev)
+        self.l_in = torch.full((B * Hq, Lq), float("-inf"), device=dev)
+        self.batched = mode == "batched"
+        self.out = {}
+
+    def project(self):
+        if self.has_proj:
+            return self.ops.kv_proj(self.x, self.wk, self.wv, self.w.Hkv)
+        return self.k, self.v
+
+    def forward(self, k, v):
+        # the travelling accumulator arrives as the identity (0, -inf) and every
+        # block's partial is folded into it by the merge kernel
+        _, _, _, o, L = self.lvx._attn_forward(self.q, k, v, False, self.w.scale, None, rounds=self.w.rounds,
+                                               mask=self.mask, acc_in=(self.o_in, self.l_in), batched=self.batched)
+        return o, L
+
+    def backward(self, k, v, o, L):
+        dq, dk, dv = self.lvx._attn_backward(self.do, self.q, k, v, o, L, False, self.w.scale, None, "flash",
+                                             rounds=self.w.rounds, mask=self.mask, batched=self.batched)
+        dx = self.ops.dx_vis(dk, dv, self.wk, self.wv) if self.has_proj else None
+        return dq, dk, dv, dx
+
+    def step(self):
+        k, v = self.project()
+        o, L = self.forward(k, v)
+        del k, v                                   # K/V are not kept for backward
+        k, v = self.project()                      # recompute
+        self.out = dict(zip(("dq", "dk", "dv", "dx"), self.backward(k, v, o, L)), o=o, L=L)
+
+
+def time_gpu(fn, iters, warmup, torch):
+    """Median-free mean duration (ms) of fn over `iters` back-to-back calls,
+    measured with events on the stream the kernels are queued on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def kernel_breakdown(layer, n_pairs, torch):
+    """Per-kernel launch durations (HIP events around repeated launches of the
+    one kernel) and their roofline fractions."""
+    ops, w = layer.ops, layer.w
+    f = flops(w, n_pairs)
+    k, v = layer.project()
+    o, L = layer.forward(k, v)
+    B, Hq, Lq, D = layer.q.shape
+    Hkv, Lkv = k.shape[1], k.shape[2]
+    dev = layer.q.device
+    o_p, l_p = torch.empty_like(o), torch.empty_like(L)
+    delta = torch.empty_like(L)
+    dq_acc = torch.zeros(B, Hq, Lq, D, dtype=torch.float32, device=dev)
+    dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+    dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
+    ops.bwd_preprocess(o, layer.do, delta)
+    res = {}
+    it = 10
+    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=layer.mask), it, 3, torch)
+    res["fwd_all_rounds_one_launch"] = dict(ms=ms, tflops=f["fwd"] / ms / 1e9, frac_mfma=f["fwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+    lb = -(-Lq // w.rounds)
+    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask), it, 3, torch)
+    res["fwd_one_round"] = dict(ms=ms, tflops=f["fwd"] / w.rounds / ms / 1e9)
+    ws = torch.empty(ops.fwd_workspace_bytes(layer.q, k, lb, 4), dtype=torch.uint8, device=dev)
+    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask, kv_splits=4,
+                                  workspace=ws), it, 3, torch)
+    res["fwd_one_round_4_key_splits"] = dict(ms=ms, tflops=f["fwd"] / w.rounds / ms / 1e9)
+    ms = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq_acc, dk, dv, w.scale, mask=layer.mask),
+                  it, 3, torch)
+    res["bwd_all_rounds_one_launch"] = dict(ms=ms, tflops=f["bwd"] / ms / 1e9, frac_mfma=f["bwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+    merge_bytes = (3 * D * 2 + 3 * 4) * B * Hq * Lq
+    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L), it, 3, torch)
+    res["merge_all_rounds_one_launch"] = dict(ms=ms, gbs=merge_bytes / ms / 1e6, frac_hbm=merge_bytes / ms / 1e6 / PEAK_HBM_GBS)
+    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L, 0, lb), it, 3, torch)
+    res["merge_one_round"] = dict(ms=ms, gbs=merge_bytes / w.rounds / ms / 1e6)
+    pre_bytes = (2 * D * 2 + 4) * B * Hq * Lq
+    ms = time_gpu(lambda: ops.bwd_preprocess(o, layer.do, delta), it, 3, torch)
+    res["preprocess"] = dict(ms=ms, gbs=pre_bytes / ms / 1e6, frac_hbm=pre_bytes / ms / 1e6 / PEAK_HBM_GBS)
+    if layer.has_proj:
+        ms = time_gpu(lambda: layer.project(), it, 3, torch)
+        res["kv_proj"] = dict(ms=ms, tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+        ms = time_gpu(lambda: ops.dx_vis(dk, dv, layer.wk, layer.wv), it, 3, torch)
+        res["dx_vis"] = dict(ms=ms, tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+    for d in res.values():
+        for key in d:
+            d[key] = round(d[key], 5)
+    return res
+
+
+def cpu_baseline(w, budget_rounds=2):
+    """The oracle (the reference's PyTorch math restated) timed on this host's
+    cores on a bounded sample: the first `budget_rounds` query blocks, forward
+    + backward against the full shard, plus the K/V projection twice and
+    dX_vis at full size."""
+    import torch
+    from oracle import lvx_oracle as orc
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    t = w.tensors
+    lb = -(-w.Lq // w.rounds)
+    rows = min(w.Lq, lb * budget_rounds)
+    q, do = t["q"][:, :, :rows], t["do"][:, :, :rows]
+
+    def run():
+        if w.Dm:
+            k, v = orc.kv_project(t["x_vis"], t["w_k"], t["w_v"], w.Hkv)
+            k, v = orc.kv_project(t["x_vis"], t["w_k"], t["w_v"], w.Hkv)
+        else:
+            k, v = t["k"], t["v"]
+        o, lse = orc.round_loop_forward(q, k, v, w.scale, budget_rounds)
+        dq, dk, dv = orc.attention_backward(do, q, k, v, o, lse, w.scale, rounds=budget_rounds)
+        if w.Dm:
+            orc.dx_vis(dk, dv, t["w_k"], t["w_v"])
+
+    run()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    f = flops(w, w.B * rows * w.Lkv)
+    total = f["fwd"] + f["bwd"] + 3 * f["proj"]
+    return {
+        "value": round(total / sec / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{w.name}: first {budget_rounds} of {w.rounds} query blocks ({rows} text rows) fwd+bwd vs the full "
+                  f"{w.Lkv}-token shard + K/V projection x2 + dX_vis at full size, fp32 torch on CPU, "
+                  f"median of 3 ({sec:.2f} s per pass)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--mode", default="batched", choices=["batched", "rounds"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build is a single-GPU path (no collectives, no sharding); run with --gpus 1")
+
+    import torch
+    from oracle import lvx_oracle as orc
+    from lv_xattn import _lib
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    _lib.load()
+    dev = "cuda:0"
+    w = orc.make_inputs(orc.workload(a.workload))
+    npairs = orc.n_pairs(w)
+    f = flops(w, npairs)
+    step_flops = f["fwd"] + f["bwd"] + 3 * f["proj"]    # projection, re-projection, dX_vis
+
+    layer = Layer(w, a.mode, dev)
+    for _ in range(a.warmup):
+        layer.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        layer.step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    value = step_flops / ms / 1e9
+
+    out = {
+        "metric": "cross-attn fwd+bwd TFLOP/s @ Llama-3.2-11B-V shape, 1 GPU; % bf16 MFMA peak",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded N(0,1) Q/dO, N(0,0.02) X_vis/W), random weights",
+        "config": {
+            "workload": f"{w.name}: B{w.B} Hq{w.Hq} Hkv{w.Hkv} D{w.D} Lq{w.Lq}={w.rounds}x{-(-w.Lq // w.rounds)} "
+                        f"Lkv{w.Lkv} Dm{w.Dm}; K/V projection + {w.rounds}-round fwd + merge + K/V re-projection "
+                        f"+ bwd + dX_vis",
+            "mode": a.mode, "flops_per_step": step_flops, "frac_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+            "flops_attention_only": f["fwd"] + f["bwd"],
+        },
+    }
+    if not a.no_breakdown:
+        kb = kernel_breakdown(layer, npairs, torch)
+        out["kernels"] = kb
+        dom = kb["bwd_all_rounds_one_launch"]
+        out["roofline"] = {"bound": "mfma", "kernel": "bwd_kernel<false>", "achieved": dom["tflops"],
+                           "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                           "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                           "avg_launch_ms": dom["ms"]}
+        other = Layer(w, "rounds" if a.mode == "batched" else "batched", dev)
+        ms2 = time_gpu(other.step, max(3, a.steps // 2), 2, torch)
+        out["config"]["other_mode"] = {"mode": other.mode, "ms_per_step": round(ms2, 4),
+                                       "tflops": round(step_flops / ms2 / 1e9, 2)}
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

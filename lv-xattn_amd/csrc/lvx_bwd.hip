@@ -9,15 +9,16 @@
 // kernel, and its dK^T / dV^T (128 x 32 each, fp32) stay in accumulators until
 // the end, so the sum over the q heads of the group and over all rows never
 // leaves the register file.  dQ needs all 128 tokens of the block: the waves
-// exchange dS (bf16) through LDS, wave w then forms dQ^T for head-dim columns
-// 32w..32w+31 with the matching K^T slice held in registers, and adds it to the
+// exchange dS (bf16) through LDS, wave w then forms dQ for head-dim columns
+// 32w..32w+31 with the matching K slice held in registers, and adds it to the
 // fp32 dQ accumulator in HBM with atomic adds (other token blocks add to the
-// same rows).
+// same rows).  The dQ tile is produced with the head-dim along the lanes, so an
+// atomic instruction covers whole 128-byte lines.
 //
 // Per 32-row step and wave: S and dP (2 x 8 MFMA, A = Q / dO row-major from
 // LDS), dV^T and dK^T (2 x 8 MFMA, A = dO^T / Q^T from LDS, B = P / dS straight
 // from the accumulators; the transposed tiles are staged with the row index
-// permuted to match), dQ^T (8 MFMA).  All MFMA are 32x32x16 bf16.
+// permuted to match), dQ (8 MFMA).  All MFMA are 32x32x16 bf16.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -126,7 +127,11 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     u32x4 pre[4];
     float pre_f = 0.f;   // tid < 32: LSE row, 32..63: delta row
     int pre_i = 0;       // 64..95: kv_start row, 96..127: kv_end row
-    auto prefetch = [&](int it) {
+    // token blocks of one kv head walk the (head, row tile) list from different
+    // starting points so that their dQ atomics do not all hit the same rows
+    const int it_shift = n_iter > 0 ? (int)(((int64_t)kblk * 7) % n_iter) : 0;
+    auto prefetch = [&](int it0) {
+        const int it = (it0 + it_shift) % n_iter;
         const int gi = it / n_qtiles, qt = it % n_qtiles;
         const int h = hk * p.G + gi;
         const int r0 = p.row_begin + qt * BM;
@@ -160,7 +165,8 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 
     if (n_iter > 0) prefetch(0);
 
-    for (int it = 0; it < n_iter; ++it) {
+    for (int it0 = 0; it0 < n_iter; ++it0) {
+        const int it = (it0 + it_shift) % n_iter;
         const int gi = it / n_qtiles, qt = it % n_qtiles;
         const int h = hk * p.G + gi;
         const int r0 = p.row_begin + qt * BM;
@@ -184,7 +190,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             else if (MASKED && tid < 128) end_s[tid - 96] = pre_i;
         }
         __syncthreads();
-        if (it + 1 < n_iter) prefetch(it + 1);
+        if (it0 + 1 < n_iter) prefetch(it0 + 1);
 
         // ---- S = Q K_w^T, dP = dO V_w^T : rows = text rows, cols = this wave's tokens
         f32x16 s, dp;
@@ -254,22 +260,26 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             }
         __syncthreads();
 
-        // ---- dQ^T[32w..32w+31, rows] = K^T slice (A, registers) x dS^T (B, from LDS)
+        // ---- dQ[rows, 32w..32w+31] = dS (A, from LDS) x K slice (B, registers).
+        // A lane ends up with one head-dim column and 16 text rows, so every
+        // atomic instruction covers two full 128-byte lines of dQ.
         f32x16 dq;
 #pragma unroll
         for (int v = 0; v < 16; ++v) dq[v] = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const bf16x8 bo = *reinterpret_cast<const bf16x8*>(&dSs[l32 * DSS + 16 * j + 8 * g]);
-            dq = mfma32(ktreg[j], bo, dq);
+            const bf16x8 ao = *reinterpret_cast<const bf16x8*>(&dSs[l32 * DSS + 16 * j + 8 * g]);
+            dq = mfma32(ao, ktreg[j], dq);
         }
-        const int row = r0 + l32;
-        if (row < p.row_end) {
-            float* dqp = p.dq_acc + (((int64_t)b * p.Hq + h) * p.Lq + row) * D + 32 * wave;
+        float* dqp = p.dq_acc + (((int64_t)b * p.Hq + h) * p.Lq + r0) * D + 32 * wave + l32;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) unsafeAtomicAdd(dqp + acc_row(v, g), dq[v] * p.scale);
+        for (int v = 0; v < 16; ++v) {
+            const int rl = acc_row(v, g);
+            if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (int64_t)rl * D, dq[v] * p.scale);
         }
-        __syncthreads();   // dS and the staged tiles are free again
+        // no barrier here: the next step's staging writes only touch tiles every
+        // wave finished reading before the barrier above, and dS is rewritten
+        // only after the next step's first barrier
     }
 
     // ---- epilogue: dK^T / dV^T rows = head-dim, cols = this wave's tokens
