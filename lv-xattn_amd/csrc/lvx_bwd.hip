@@ -255,8 +255,10 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             for (int e = 0; e < 4; ++e) {
                 const int v = 8 * j + 2 * e;
                 const uint32_t u = dsu[j][e];
+#ifndef LVX_EXP_NO_DSWRITE
                 dSs[acc_row(v, g) * DSS + 32 * wave + l32] = (uint16_t)(u & 0xffffu);
                 dSs[acc_row(v + 1, g) * DSS + 32 * wave + l32] = (uint16_t)(u >> 16);
+#endif
             }
         __syncthreads();
 
@@ -275,7 +277,11 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int rl = acc_row(v, g);
+#ifdef LVX_EXP_NO_ATOMICS
+            if (dq[v] == 12345.678f) dqp[(int64_t)rl * D] = 1.f;
+#else
             if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (int64_t)rl * D, dq[v] * p.scale);
+#endif
         }
         // no barrier here: the next step's staging writes only touch tiles every
         // wave finished reading before the barrier above, and dS is rewritten

@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "liblvx.so")
+LIB_PATH = os.environ.get("LVX_LIB") or os.path.join(_HERE, "liblvx.so")
 
 LVX_BF16 = 1
 
