@@ -15,10 +15,14 @@
 // same rows).  The dQ tile is produced with the head-dim along the lanes, so an
 // atomic instruction covers whole 128-byte lines.
 //
-// Per 32-row step and wave: S and dP (2 x 8 MFMA, A = Q / dO row-major from
-// LDS), dV^T and dK^T (2 x 8 MFMA, A = dO^T / Q^T from LDS, B = P / dS straight
-// from the accumulators; the transposed tiles are staged with the row index
-// permuted to match), dQ (8 MFMA).  All MFMA are 32x32x16 bf16.
+// Per 32-row step and wave (all MFMA are 32x32x16 bf16):
+//   S, dP        2 x 8 MFMA   A = Q / dO rows from LDS (16-byte reads)
+//   dV^T, dK^T   2 x 8 MFMA   A = dO^T / Q^T, read from the SAME row-major LDS
+//                             tiles with the transposing LDS read; B = P / dS
+//                             straight from the accumulators (the transposing
+//                             read is addressed in the accumulator's row order)
+//   dQ           8 MFMA       A = dS, read transposed from the dS^T tile the
+//                             waves wrote (8-byte writes), B = K slice
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -29,22 +33,20 @@ namespace {
 constexpr int D = 128;
 constexpr int BN = 128;       // visual tokens per work-group
 constexpr int BM = 32;        // text rows per step
-constexpr int QS = D + 8;     // row stride of the row-major Q / dO tiles
-constexpr int TS = BM + 8;    // row stride of the transposed Q^T / dO^T tiles
-constexpr int DSS = BN + 8;   // row stride of the dS tile
-constexpr int KTS = BN + 8;   // row stride of the K^T staging tile (prologue only)
+constexpr int QS = D + 8;     // row stride of the Q / dO tiles (68 dwords: 16-byte row reads conflict-free)
+constexpr int DSS = BM + 4;   // row stride of the dS^T tile [token][row] (18 dwords)
+constexpr int KPS = D + 8;    // row stride of the K tile staged once in the prologue
 
 constexpr int OFF_Q = 0;
 constexpr int OFF_DO = OFF_Q + BM * QS;
-constexpr int OFF_QT = OFF_DO + BM * QS;
-constexpr int OFF_DOT = OFF_QT + D * TS;
-constexpr int OFF_DS = OFF_DOT + D * TS;
-constexpr int TILE_ELEMS = OFF_DS + BM * DSS;
-static_assert(D * KTS <= OFF_DS, "K^T staging must fit under the dS tile");
+constexpr int OFF_DS = OFF_DO + BM * QS;
+constexpr int LOOP_ELEMS = OFF_DS + BN * DSS;
+constexpr int PRO_ELEMS = BN * KPS;
+constexpr int SMEM_ELEMS = LOOP_ELEMS > PRO_ELEMS ? LOOP_ELEMS : PRO_ELEMS;
 
 template <bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t smem[TILE_ELEMS];
+    __shared__ __attribute__((aligned(16))) uint16_t smem[SMEM_ELEMS];
     __shared__ __attribute__((aligned(16))) float lse_s[BM];
     __shared__ __attribute__((aligned(16))) float delta_s[BM];
     __shared__ __attribute__((aligned(16))) int start_s[BM];
@@ -65,17 +67,18 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     const int kvb = kblk * BN;
     const int my_kv = kvb + 32 * wave + l32;
     const bool kv_valid = my_kv < kv_len;
+    const bool tail_block = kvb + BN > kv_len;
 
     uint16_t* Qs = smem + OFF_Q;
     uint16_t* dOs = smem + OFF_DO;
-    uint16_t* QT = smem + OFF_QT;
-    uint16_t* dOT = smem + OFF_DOT;
-    uint16_t* dSs = smem + OFF_DS;
+    uint16_t* dST = smem + OFF_DS;
 
     const uint16_t* kbase = p.k + b * p.ks.b + hk * p.ks.h;
     const uint16_t* vbase = p.v + b * p.vs.b + hk * p.vs.h;
 
-    // ---- prologue: K, V rows of this wave as B operands; K^T slice as A operand
+    // ---- prologue: K, V rows of this wave as B operands (contraction over d),
+    //      and the K slice [tokens of the block][32w..32w+31] as B operand for dQ
+    //      (contraction over the tokens)
     bf16x8 kreg[8], vreg[8], ktreg[8];
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
@@ -83,28 +86,18 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         vreg[kk] = as_bf16x8(ldg16(vbase + (int64_t)my_kv * p.vs.s + kk * 16 + g * 8, kv_valid));
     }
     {
-        // stage K^T[d][token] of the whole 128-token block (natural token order)
-        uint16_t* KT = smem;
+        uint16_t* Kp = smem;
 #pragma unroll
-        for (int rep = 0; rep < 2; ++rep) {
-            const int blk = tid + 256 * rep;        // 512 blocks of 4 tokens x 8 columns
-            const int chunk = blk & 15, group = blk >> 4;
-            u32x4 r[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int kv = kvb + 4 * group + i;
-                r[i] = ldg16(kbase + (int64_t)kv * p.ks.s + chunk * 8, kv < kv_len);
-            }
-            u32x2 t8[8];
-            transpose_4x8(r, t8);
-#pragma unroll
-            for (int d = 0; d < 8; ++d)
-                *reinterpret_cast<u32x2*>(&KT[(chunk * 8 + d) * KTS + 4 * group]) = t8[d];
+        for (int i = 0; i < 8; ++i) {
+            const int c = tid + 256 * i;
+            const int kv = kvb + (c >> 4);
+            *reinterpret_cast<u32x4*>(&Kp[(c >> 4) * KPS + (c & 15) * 8]) =
+                ldg16(kbase + (int64_t)kv * p.ks.s + (c & 15) * 8, kv < kv_len);
         }
         __syncthreads();
+        const int off = tr_lane_offset(lane, KPS, false) + 32 * wave;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            ktreg[j] = *reinterpret_cast<const bf16x8*>(&KT[(32 * wave + l32) * KTS + 16 * j + 8 * g]);
+        for (int j = 0; j < 8; ++j) ktreg[j] = lds_operand_tr(&Kp[off + 16 * j * KPS], 4 * KPS);
         __syncthreads();
     }
 
@@ -123,6 +116,11 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     const int st = tid & 127;
     const int s_chunk = st & 15, s_group = st >> 4;
     const bool is_do = tid >= 128;
+    uint16_t* stage_dst = (is_do ? dOs : Qs) + 4 * s_group * QS + s_chunk * 8;
+
+    // per-lane offsets of the transposing operand reads
+    const int off_qT = tr_lane_offset(lane, QS, true);     // Q^T / dO^T, rows in accumulator order
+    const int off_dsT = tr_lane_offset(lane, DSS, false);  // dS from dS^T, tokens in natural order
 
     u32x4 pre[4];
     float pre_f = 0.f;   // tid < 32: LSE row, 32..63: delta row
@@ -171,24 +169,13 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         const int h = hk * p.G + gi;
         const int r0 = p.row_begin + qt * BM;
 
-        // ---- stage this step's Q / dO tile, row-major and transposed
-        {
-            uint16_t* rm = is_do ? dOs : Qs;
-            uint16_t* tr = is_do ? dOT : QT;
+        // ---- stage this step's Q / dO tile (row-major only)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<u32x4*>(&rm[(4 * s_group + i) * QS + s_chunk * 8]) = pre[i];
-            u32x2 t8[8];
-            transpose_4x8(pre, t8);
-            const int pos = swap23(4 * s_group);
-#pragma unroll
-            for (int d = 0; d < 8; ++d)
-                *reinterpret_cast<u32x2*>(&tr[(s_chunk * 8 + d) * TS + pos]) = t8[d];
-            if (tid < 32) lse_s[tid] = pre_f;
-            else if (tid < 64) delta_s[tid - 32] = pre_f;
-            else if (MASKED && tid < 96) start_s[tid - 64] = pre_i;
-            else if (MASKED && tid < 128) end_s[tid - 96] = pre_i;
-        }
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(stage_dst + i * QS) = pre[i];
+        if (tid < 32) lse_s[tid] = pre_f;
+        else if (tid < 64) delta_s[tid - 32] = pre_f;
+        else if (MASKED && tid < 96) start_s[tid - 64] = pre_i;
+        else if (MASKED && tid < 128) end_s[tid - 96] = pre_i;
         __syncthreads();
         if (it0 + 1 < n_iter) prefetch(it0 + 1);
 
@@ -204,7 +191,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             dp = mfma32(ad, vreg[kk], dp);
         }
 
-        // ---- P and dS (register v of lane-half g is text row 8*(v/4)+4g+(v%4))
+        // ---- P and scale*dS (register v of lane-half g is text row 8*(v/4)+4g+(v%4))
 #pragma unroll
         for (int vg = 0; vg < 4; ++vg) {
             const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[8 * vg + 4 * g]);
@@ -212,15 +199,28 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int v = 4 * vg + r;
-                float pv = __builtin_amdgcn_exp2f(fmaf(s[v], c, -l4[r]));
-                bool vis = kv_valid;
-                if (MASKED) {
-                    const int q_local = 8 * vg + 4 * g + r;
-                    vis = vis && my_kv >= start_s[q_local] && my_kv < end_s[q_local];
-                }
-                pv = vis ? pv : 0.f;
+                const float pv = __builtin_amdgcn_exp2f(fmaf(s[v], c, -l4[r]));
                 s[v] = pv;
-                dp[v] = pv * (dp[v] - d4[r]);
+                dp[v] = pv * p.scale * (dp[v] - d4[r]);
+            }
+        }
+        if (MASKED) {
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                const int* sp = &start_s[8 * vg + 4 * g];
+                const int* ep = &end_s[8 * vg + 4 * g];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool vis = kv_valid && my_kv >= sp[r] && my_kv < ep[r];
+                    s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
+                    dp[4 * vg + r] = vis ? dp[4 * vg + r] : 0.f;
+                }
+            }
+        } else if (tail_block) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                s[v] = kv_valid ? s[v] : 0.f;
+                dp[v] = kv_valid ? dp[v] : 0.f;
             }
         }
         bf16x8 pb[2], dsb[2];
@@ -237,32 +237,29 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             dsb[j] = as_bf16x8(dsu[j]);
         }
 
-        // ---- dV_w^T += dO^T P,  dK_w^T += Q^T dS  (contraction over the 32 text rows)
+        // ---- hand scale*dS to the other waves: dST[token of the block][text row]
+        {
+            uint16_t* dsp = &dST[(32 * wave + l32) * DSS + 4 * g];
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                const u32x2 w = {dsu[vg >> 1][2 * (vg & 1)], dsu[vg >> 1][2 * (vg & 1) + 1]};
+                *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
+            }
+        }
+
+        // ---- dV_w^T += dO^T P,  dK_w^T += Q^T (scale*dS)  (contraction over the 32 text rows)
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(&dOT[(dt * 32 + l32) * TS + 16 * j + 8 * g]);
-                const bf16x8 a2 = *reinterpret_cast<const bf16x8*>(&QT[(dt * 32 + l32) * TS + 16 * j + 8 * g]);
+                const bf16x8 a1 = lds_operand_tr(&dOs[off_qT + 16 * j * QS + dt * 32], 8 * QS);
+                const bf16x8 a2 = lds_operand_tr(&Qs[off_qT + 16 * j * QS + dt * 32], 8 * QS);
                 dv[dt] = mfma32(a1, pb[j], dv[dt]);
                 dk[dt] = mfma32(a2, dsb[j], dk[dt]);
             }
-
-        // ---- hand dS to the other waves: dSs[text row][token of the block]
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int v = 8 * j + 2 * e;
-                const uint32_t u = dsu[j][e];
-#ifndef LVX_EXP_NO_DSWRITE
-                dSs[acc_row(v, g) * DSS + 32 * wave + l32] = (uint16_t)(u & 0xffffu);
-                dSs[acc_row(v + 1, g) * DSS + 32 * wave + l32] = (uint16_t)(u >> 16);
-#endif
-            }
         __syncthreads();
 
-        // ---- dQ[rows, 32w..32w+31] = dS (A, from LDS) x K slice (B, registers).
+        // ---- dQ[rows, 32w..32w+31] = (scale*dS) (A, transposed read) x K slice (B, registers).
         // A lane ends up with one head-dim column and 16 text rows, so every
         // atomic instruction covers two full 128-byte lines of dQ.
         f32x16 dq;
@@ -270,7 +267,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         for (int v = 0; v < 16; ++v) dq[v] = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const bf16x8 ao = *reinterpret_cast<const bf16x8*>(&dSs[l32 * DSS + 16 * j + 8 * g]);
+            const bf16x8 ao = lds_operand_tr(&dST[off_dsT + 16 * j * DSS], 4 * DSS);
             dq = mfma32(ao, ktreg[j], dq);
         }
         float* dqp = p.dq_acc + (((int64_t)b * p.Hq + h) * p.Lq + r0) * D + 32 * wave + l32;
@@ -280,11 +277,11 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 #ifdef LVX_EXP_NO_ATOMICS
             if (dq[v] == 12345.678f) dqp[(int64_t)rl * D] = 1.f;
 #else
-            if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (int64_t)rl * D, dq[v] * p.scale);
+            if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (int64_t)rl * D, dq[v]);
 #endif
         }
         // no barrier here: the next step's staging writes only touch tiles every
-        // wave finished reading before the barrier above, and dS is rewritten
+        // wave finished reading before the barrier above, and dS^T is rewritten
         // only after the next step's first barrier
     }
 
@@ -302,7 +299,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
                     f32x4 bb = *reinterpret_cast<f32x4*>(dvp + d);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        a[r] += dk[dt][4 * vg + r] * p.scale;
+                        a[r] += dk[dt][4 * vg + r];
                         bb[r] += dv[dt][4 * vg + r];
                     }
                     *reinterpret_cast<f32x4*>(dkp + d) = a;
@@ -317,8 +314,8 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
                     u32x2 a, bb;
-                    a[0] = pack_bf16(dk[dt][4 * vg] * p.scale, dk[dt][4 * vg + 1] * p.scale);
-                    a[1] = pack_bf16(dk[dt][4 * vg + 2] * p.scale, dk[dt][4 * vg + 3] * p.scale);
+                    a[0] = pack_bf16(dk[dt][4 * vg], dk[dt][4 * vg + 1]);
+                    a[1] = pack_bf16(dk[dt][4 * vg + 2], dk[dt][4 * vg + 3]);
                     bb[0] = pack_bf16(dv[dt][4 * vg], dv[dt][4 * vg + 1]);
                     bb[1] = pack_bf16(dv[dt][4 * vg + 2], dv[dt][4 * vg + 3]);
                     *reinterpret_cast<u32x2*>(dkp + d) = a;

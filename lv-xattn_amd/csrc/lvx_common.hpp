@@ -69,6 +69,39 @@ __device__ __forceinline__ void transpose_4x8(const u32x4 r[4], u32x2 out[8]) {
     }
 }
 
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef s16x4 __attribute__((address_space(3)))* lds_s16x4_ptr;
+
+// ds_read_b64_tr_b16: every lane supplies the LDS address of an 8-byte word
+// (4 x 16 bit).  Within each group of 16 lanes, lane i receives element (i & 3)
+// of the words addressed by lanes (i >> 2), (i >> 2) + 4, + 8, + 12.  Pointing
+// the lane quad q of a group at row k0 + q of a tile T[k][m] (m contiguous,
+// lane q*4 + t at columns m0 + 4t .. 4t+3) hands lane i the four values
+// T[k0 .. k0+3][m0 + i]: an MFMA operand whose contraction index runs down the
+// rows of a tile stored with the OTHER index contiguous, with no transposed copy.
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
+    s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p);
+    return __builtin_bit_cast(u32x2, r);
+}
+
+// Per-lane element offset into T[k][m] (row stride `stride`) for a transposing
+// operand read of a 32(m) x 16(k) MFMA operand; the second half of the operand
+// (slots e = 4..7) is `half_rows` rows further down.
+//   natural order : slot (g, e) <-> k = 8g + e          -> half_rows = 4
+//   permuted order: slot (g, e) <-> k = 8(e/4) + 4g + e%4 -> half_rows = 8
+// (the permuted order is the one an accumulator tile has when it is fed back
+// as the other operand).
+__device__ __forceinline__ int tr_lane_offset(int lane, int stride, bool permuted) {
+    const int r = (lane & 15) >> 2, t = lane & 3, u = (lane >> 4) & 1, g = lane >> 5;
+    return ((permuted ? 4 * g : 8 * g) + r) * stride + 16 * u + 4 * t;
+}
+
+__device__ __forceinline__ bf16x8 lds_operand_tr(const uint16_t* p, int half_offset) {
+    const u32x2 a = lds_read_tr16(p), b = lds_read_tr16(p + half_offset);
+    const u32x4 u = {a[0], a[1], b[0], b[1]};
+    return as_bf16x8(u);
+}
+
 // Work-groups are dealt to the 8 XCDs round-robin by linear id.  Remap so that
 // each XCD receives one contiguous range of the work list: neighbours in the
 // list (which share K/V or Q tiles) then share that XCD's L2.

@@ -14,12 +14,15 @@
 //                    the two lane halves; rescaling O is a per-lane scalar
 //   O^T[d, row]   += V^T_tile (A, from LDS) x  P^T (B, straight from the S^T
 //                    accumulators: register v of lane-half g is key
-//                    8*(v/4)+4*g+(v%4), and V^T is staged with its key index
-//                    permuted the same way, so P never visits LDS)
-// K is staged row-major [64][128+8], V transposed [128][64+8] (transposed in
-// registers on the way in); the +8 element pad makes the 16-byte operand reads
-// of 16 consecutive lanes hit 64 distinct banks.  The next tile's global loads
-// are in flight while the current one is consumed.
+//                    8*(v/4)+4*g+(v%4); the V^T operand is fetched from the
+//                    row-major V tile with the transposing LDS read, addressed
+//                    in that same key order, so P never visits LDS and V is
+//                    never transposed in memory)
+// K and V are both staged row-major: K [64][128+8] (68-dword rows: the 16-byte
+// operand reads of 16 consecutive lanes hit 64 distinct banks), V [64][128+16]
+// (72-dword rows: the 8 rows x 16 dwords a transposing read touches tile the
+// banks twice).  The next tile's global loads are in flight while the current
+// one is consumed.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -30,13 +33,13 @@ namespace {
 constexpr int D = 128;
 constexpr int BN = 64;        // keys per tile
 constexpr int KS = D + 8;     // K tile row stride (elements)
-constexpr int VS = BN + 8;    // V^T tile row stride (elements)
+constexpr int VS = D + 16;    // V tile row stride (elements)
 constexpr int BIG = 0x3fffffff;
 
 template <bool MASKED>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * VS];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * VS];
     __shared__ int red[4][4];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
@@ -102,9 +105,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
     const uint16_t* kbase = p.k + b * p.ks.b + hk * p.ks.h;
     const uint16_t* vbase = p.v + b * p.vs.b + hk * p.vs.h;
-    // V staging: each thread owns a 4-key x 8-column block of the tile
-    const int vchunk = (lane & 7) + 8 * (wave & 1);
-    const int vgroup = (lane >> 3) + 8 * (wave >> 1);
+    const int off_vT = tr_lane_offset(lane, VS, true);   // V^T operand, keys in accumulator order
 
     u32x4 kpre[4], vpre[4];
     auto prefetch = [&](int kv0) {
@@ -116,8 +117,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int kv = kv0 + 4 * vgroup + i;
-            vpre[i] = ldg16(vbase + (int64_t)kv * p.vs.s + vchunk * 8, kv < kv_hi);
+            const int c = tid + 256 * i;
+            const int kv = kv0 + (c >> 4);
+            vpre[i] = ldg16(vbase + (int64_t)kv * p.vs.s + (c & 15) * 8, kv < kv_hi);
         }
     };
 
@@ -140,14 +142,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int i = 0; i < 4; ++i) {
             const int cidx = tid + 256 * i;
             *reinterpret_cast<u32x4*>(&Ks[(cidx >> 4) * KS + (cidx & 15) * 8]) = kpre[i];
-        }
-        {
-            u32x2 vt[8];
-            transpose_4x8(vpre, vt);
-            const int pos = swap23(4 * vgroup);
-#pragma unroll
-            for (int d = 0; d < 8; ++d)
-                *reinterpret_cast<u32x2*>(&Vt[(vchunk * 8 + d) * VS + pos]) = vt[d];
+            *reinterpret_cast<u32x4*>(&Vs[(cidx >> 4) * VS + (cidx & 15) * 8]) = vpre[i];
         }
         __syncthreads();
         if (t + 1 < t_end) prefetch(kv0 + BN);
@@ -215,7 +210,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Vt[(dt * 32 + l32) * VS + j * 16 + g * 8]);
+                const bf16x8 a = lds_operand_tr(&Vs[off_vT + 16 * j * VS + dt * 32], 8 * VS);
                 acc[dt] = mfma32(a, pb[j], acc[dt]);
             }
     }

@@ -4,11 +4,13 @@
 // v_mfma_f32_32x32x16_bf16, bf16 output.
 //
 // A work-group computes a 128 x 128 tile of C with 4 waves (64 x 64 each, 2 x 2
-// MFMA tiles), stepping 64 along the contraction.  Both operand tiles are
-// staged in LDS with the contraction index contiguous ([128][64+8]); an operand
-// whose memory order has the other index contiguous is transposed in registers
-// on its way in.  The MFMA computes C^T (A operand = rows of the B tile), so a
-// lane ends up with 4 consecutive columns of one C row and stores 8 bytes.
+// MFMA tiles), stepping 64 along the contraction.  An operand whose memory has
+// the contraction index contiguous is staged as [128][64+8] and read with
+// 16-byte LDS reads; an operand whose memory has the OTHER index contiguous is
+// staged exactly as it lies in memory, [64 k][128+32], and read with the
+// transposing LDS read - nothing is transposed on the way in.  The MFMA
+// computes C^T (A operand = rows of the B tile), so a lane ends up with 4
+// consecutive columns of one C row and stores 8 bytes.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -17,25 +19,23 @@ namespace lvx {
 namespace {
 
 constexpr int TM = 128, TN = 128, BK = 64;
-constexpr int LS = BK + 8;   // LDS row stride (elements)
+constexpr int LS = BK + 8;     // row stride of a [row][k] tile (36 dwords)
+constexpr int LT = TM + 32;    // row stride of a [k][row] tile (80 dwords)
+constexpr int TILE_ELEMS = (TM * LS > BK * LT) ? TM * LS : BK * LT;
 
-// Load the [128 rows][64 k] tile starting at (r0, k0) into 4 registers of 16 B.
-// CONTIG_K: memory is [row][k]; otherwise memory is [k][row].
+// Fetch the tile covering rows r0..r0+127 and k0..k0+63 into 4 x 16 bytes.
+// ROW_CONTIG: memory is [k][row]; otherwise memory is [row][k].
 template <bool ROW_CONTIG>
 __device__ __forceinline__ void tile_load(u32x4 pre[4], const uint16_t* base, int64_t ld, int r0, int k0,
                                           int R, int K, int tid) {
-    if (!ROW_CONTIG) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i;
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + 256 * i;
+        if (!ROW_CONTIG) {
             const int r = r0 + (c >> 3), k = k0 + (c & 7) * 8;
             pre[i] = ldg16(base + (int64_t)r * ld + k, r < R && k < K);
-        }
-    } else {
-        const int rchunk = tid & 15, kgroup = tid >> 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int k = k0 + 4 * kgroup + i, r = r0 + 8 * rchunk;
+        } else {
+            const int k = k0 + (c >> 4), r = r0 + (c & 15) * 8;
             pre[i] = ldg16(base + (int64_t)k * ld + r, k < K && r < R);
         }
     }
@@ -43,26 +43,28 @@ __device__ __forceinline__ void tile_load(u32x4 pre[4], const uint16_t* base, in
 
 template <bool ROW_CONTIG>
 __device__ __forceinline__ void tile_store(const u32x4 pre[4], uint16_t* lds, int tid) {
-    if (!ROW_CONTIG) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i;
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + 256 * i;
+        if (!ROW_CONTIG)
             *reinterpret_cast<u32x4*>(&lds[(c >> 3) * LS + (c & 7) * 8]) = pre[i];
-        }
-    } else {
-        const int rchunk = tid & 15, kgroup = tid >> 4;
-        u32x2 t8[8];
-        transpose_4x8(pre, t8);
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-            *reinterpret_cast<u32x2*>(&lds[(8 * rchunk + r) * LS + 4 * kgroup]) = t8[r];
+        else
+            *reinterpret_cast<u32x4*>(&lds[(c >> 4) * LT + (c & 15) * 8]) = pre[i];
     }
+}
+
+// MFMA operand for tile rows row0..row0+31 and k-step kk (16 values of k).
+template <bool ROW_CONTIG>
+__device__ __forceinline__ bf16x8 tile_operand(const uint16_t* lds, int row0, int kk, int lane, int tr_off) {
+    if (!ROW_CONTIG)
+        return *reinterpret_cast<const bf16x8*>(&lds[(row0 + (lane & 31)) * LS + kk * 16 + (lane >> 5) * 8]);
+    return lds_operand_tr(&lds[tr_off + row0 + kk * 16 * LT], 4 * LT);
 }
 
 template <bool A_MCONTIG, bool B_NCONTIG>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[TM * LS];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[TN * LS];
+    __shared__ __attribute__((aligned(16))) uint16_t As[TILE_ELEMS];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[TILE_ELEMS];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
@@ -75,6 +77,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wm = wave & 1, wn = wave >> 1;
+    const int tr_off = tr_lane_offset(lane, LT, false);
 
     f32x16 acc[2][2];   // [n tile][m tile]
 #pragma unroll
@@ -108,8 +111,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
             bf16x8 am[2], bn[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                am[t] = *reinterpret_cast<const bf16x8*>(&As[(64 * wm + 32 * t + l32) * LS + kk * 16 + g * 8]);
-                bn[t] = *reinterpret_cast<const bf16x8*>(&Bs[(64 * wn + 32 * t + l32) * LS + kk * 16 + g * 8]);
+                am[t] = tile_operand<A_MCONTIG>(As, 64 * wm + 32 * t, kk, lane, tr_off);
+                bn[t] = tile_operand<B_NCONTIG>(Bs, 64 * wn + 32 * t, kk, lane, tr_off);
             }
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt)
