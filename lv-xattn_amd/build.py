@@ -27,6 +27,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results in arch VGPRs (the VALU reads them without copies); the
+    # register allocator then parks long-lived MFMA operands in AGPRs instead
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -47,10 +47,14 @@ constexpr int SMEM_ELEMS = LOOP_ELEMS > PRO_ELEMS ? LOOP_ELEMS : PRO_ELEMS;
 template <bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     __shared__ __attribute__((aligned(16))) uint16_t smem[SMEM_ELEMS];
-    __shared__ __attribute__((aligned(16))) float lse_s[BM];
-    __shared__ __attribute__((aligned(16))) float delta_s[BM];
-    __shared__ __attribute__((aligned(16))) int start_s[BM];
-    __shared__ __attribute__((aligned(16))) int end_s[BM];
+    // per-row metadata of the staged tile: [0,32) LSE*log2e, [32,64) delta,
+    // [64,96) kv_start, [96,128) kv_end (raw 32-bit words)
+    __shared__ u32x4 meta_s4[BM];
+    uint32_t* meta_s = reinterpret_cast<uint32_t*>(meta_s4);
+    const u32x4* lse_s4 = meta_s4;            // 8 x 16 bytes each
+    const u32x4* delta_s4 = meta_s4 + 8;
+    const u32x4* start_s4 = meta_s4 + 16;
+    const u32x4* end_s4 = meta_s4 + 24;
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
@@ -118,18 +122,23 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     const bool is_do = tid >= 128;
     uint16_t* stage_dst = (is_do ? dOs : Qs) + 4 * s_group * QS + s_chunk * 8;
 
+    const int dq_lane = 4 * g * D + 32 * wave + l32;   // this lane's element offset inside a dQ tile
+
     // per-lane offsets of the transposing operand reads
     const int off_qT = tr_lane_offset(lane, QS, true);     // Q^T / dO^T, rows in accumulator order
     const int off_dsT = tr_lane_offset(lane, DSS, false);  // dS from dS^T, tokens in natural order
 
     u32x4 pre[4];
-    float pre_f = 0.f;   // tid < 32: LSE row, 32..63: delta row
-    int pre_i = 0;       // 64..95: kv_start row, 96..127: kv_end row
+    uint32_t pre_m = 0;
+    // Every load below is unconditional: rows past the window are clamped to its
+    // last row (their LSE is forced to +inf, so P = 0 and nothing they carry
+    // reaches a result), and the step after the last one re-reads the last.
+    const int meta_kind = (tid >> 5) & 3;    // 0 LSE, 1 delta, 2 kv_start, 3 kv_end
     // token blocks of one kv head walk the (head, row tile) list from different
     // starting points so that their dQ atomics do not all hit the same rows
     const int it_shift = n_iter > 0 ? (int)(((int64_t)kblk * 7) % n_iter) : 0;
     auto prefetch = [&](int it0) {
-        const int it = (it0 + it_shift) % n_iter;
+        const int it = (min(it0, n_iter - 1) + it_shift) % n_iter;
         const int gi = it / n_qtiles, qt = it % n_qtiles;
         const int h = hk * p.G + gi;
         const int r0 = p.row_begin + qt * BM;
@@ -138,27 +147,23 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         const int64_t rs = is_do ? p.dos.s : p.qs.s;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int row = r0 + 4 * s_group + i;
-            pre[i] = ldg16(base + (int64_t)row * rs + s_chunk * 8, row < p.row_end);
+            const int row = min(r0 + 4 * s_group + i, p.row_end - 1);
+            pre[i] = *reinterpret_cast<const u32x4*>(base + (int64_t)row * rs + s_chunk * 8);
         }
-        if (tid < 64) {
-            const int row = r0 + (tid & 31);
-            const bool ok = row < p.row_end;
-            const int64_t off = ((int64_t)b * p.Hq + h) * p.Lq + row;
-            if (tid < 32) {
-                const float l = ok ? p.lse[off] : -INFINITY;
-                // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
-                pre_f = (l == -INFINITY) ? INFINITY : l * LOG2E;
-            } else {
-                pre_f = ok ? p.delta[off] : 0.f;
-            }
-        } else if (MASKED && tid < 128) {
-            const int row = r0 + (tid & 31);
-            const bool ok = row < p.row_end;
-            const int64_t off = (int64_t)b * p.Lq + row;
-            if (tid < 96) pre_i = ok ? p.kv_start[off] : 0;
-            else pre_i = ok ? p.kv_end[off] : 0;
-        }
+        const int mrow = r0 + (tid & 31);
+        const bool ok = mrow < p.row_end;
+        const int crow = min(mrow, p.row_end - 1);
+        const int64_t off_bh = ((int64_t)b * p.Hq + h) * p.Lq + crow;
+        const int64_t off_b = (int64_t)b * p.Lq + crow;
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(p.lse) + off_bh;
+        if (meta_kind == 1) src = reinterpret_cast<const uint32_t*>(p.delta) + off_bh;
+        if (MASKED && meta_kind == 2) src = reinterpret_cast<const uint32_t*>(p.kv_start) + off_b;
+        if (MASKED && meta_kind == 3) src = reinterpret_cast<const uint32_t*>(p.kv_end) + off_b;
+        const uint32_t raw = *src;
+        const float l = __uint_as_float(raw);
+        // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
+        const float lt = (!ok || l == -INFINITY) ? INFINITY : l * LOG2E;
+        pre_m = meta_kind == 0 ? __float_as_uint(lt) : (ok ? raw : 0u);
     };
 
     if (n_iter > 0) prefetch(0);
@@ -172,12 +177,9 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         // ---- stage this step's Q / dO tile (row-major only)
 #pragma unroll
         for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(stage_dst + i * QS) = pre[i];
-        if (tid < 32) lse_s[tid] = pre_f;
-        else if (tid < 64) delta_s[tid - 32] = pre_f;
-        else if (MASKED && tid < 96) start_s[tid - 64] = pre_i;
-        else if (MASKED && tid < 128) end_s[tid - 96] = pre_i;
+        meta_s[tid & 127] = pre_m;     // both halves of the group write the same words
         __syncthreads();
-        if (it0 + 1 < n_iter) prefetch(it0 + 1);
+        prefetch(it0 + 1);
 
         // ---- S = Q K_w^T, dP = dO V_w^T : rows = text rows, cols = this wave's tokens
         f32x16 s, dp;
@@ -194,8 +196,8 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         // ---- P and scale*dS (register v of lane-half g is text row 8*(v/4)+4g+(v%4))
 #pragma unroll
         for (int vg = 0; vg < 4; ++vg) {
-            const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[8 * vg + 4 * g]);
-            const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[8 * vg + 4 * g]);
+            const f32x4 l4 = __builtin_bit_cast(f32x4, lse_s4[2 * vg + g]);
+            const f32x4 d4 = __builtin_bit_cast(f32x4, delta_s4[2 * vg + g]);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int v = 4 * vg + r;
@@ -207,11 +209,11 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         if (MASKED) {
 #pragma unroll
             for (int vg = 0; vg < 4; ++vg) {
-                const int* sp = &start_s[8 * vg + 4 * g];
-                const int* ep = &end_s[8 * vg + 4 * g];
+                const u32x4 sp = start_s4[2 * vg + g];
+                const u32x4 ep = end_s4[2 * vg + g];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool vis = kv_valid && my_kv >= sp[r] && my_kv < ep[r];
+                    const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
                     s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
                     dp[4 * vg + r] = vis ? dp[4 * vg + r] : 0.f;
                 }
@@ -270,15 +272,16 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             const bf16x8 ao = lds_operand_tr(&dST[off_dsT + 16 * j * DSS], 4 * DSS);
             dq = mfma32(ao, ktreg[j], dq);
         }
-        float* dqp = p.dq_acc + (((int64_t)b * p.Hq + h) * p.Lq + r0) * D + 32 * wave + l32;
+        float* dqp = p.dq_acc + (((int64_t)b * p.Hq + h) * p.Lq + r0) * D;   // uniform
+        if (r0 + BM <= p.row_end) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int rl = acc_row(v, g);
-#ifdef LVX_EXP_NO_ATOMICS
-            if (dq[v] == 12345.678f) dqp[(int64_t)rl * D] = 1.f;
-#else
-            if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (int64_t)rl * D, dq[v]);
-#endif
+            for (int v = 0; v < 16; ++v) unsafeAtomicAdd(dqp + (dq_lane + (8 * (v >> 2) + (v & 3)) * D), dq[v]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int rl = acc_row(v, g);
+                if (r0 + rl < p.row_end) unsafeAtomicAdd(dqp + (dq_lane + (8 * (v >> 2) + (v & 3)) * D), dq[v]);
+            }
         }
         // no barrier here: the next step's staging writes only touch tiles every
         // wave finished reading before the barrier above, and dS^T is rewritten
