@@ -114,7 +114,8 @@ def kernel_breakdown(layer, n_pairs, torch):
     dev = layer.q.device
     o_p, l_p = torch.empty_like(o), torch.empty_like(L)
     delta = torch.empty_like(L)
-    dq_acc = torch.zeros(B, Hq, Lq, D, dtype=torch.float32, device=dev)
+    dq = torch.empty(B, Hq, Lq, D, dtype=torch.bfloat16, device=dev)
+    bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq), dtype=torch.uint8, device=dev)
     dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
     dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
     ops.bwd_preprocess(o, layer.do, delta)
@@ -129,8 +130,8 @@ def kernel_breakdown(layer, n_pairs, torch):
     ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask, kv_splits=4,
                                   workspace=ws), it, 3, torch)
     res["fwd_one_round_4_key_splits"] = dict(ms=ms, tflops=f["fwd"] / w.rounds / ms / 1e9)
-    ms = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq_acc, dk, dv, w.scale, mask=layer.mask),
-                  it, 3, torch)
+    ms = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask,
+                                  workspace=bws), it, 3, torch)
     res["bwd_all_rounds_one_launch"] = dict(ms=ms, tflops=f["bwd"] / ms / 1e9, frac_mfma=f["bwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
     merge_bytes = (3 * D * 2 + 3 * 4) * B * Hq * Lq
     ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L), it, 3, torch)

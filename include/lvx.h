@@ -106,18 +106,23 @@ int lvx_bwd_preprocess(const lvx_attn_shape* shape, const lvx_tensor* o, const l
 /*
  * Backward of the selected text rows against the whole local shard, from the
  * saved (finally merged) LSE and delta.  Replaces `_bwd_kernel`
- * (lv_xattn/flash_attn_kernels.py:364-640, 677-819; launcher :904-1020) and the
- * host-side `dk += dk_delta; dv += dv_delta` of lv_xattn/attn.py:523-524.
- *   dq_acc : fp32 [B, Hq, Lq, D] contiguous; contributions are ADDED (atomic),
- *            the caller zeroes it once before the first round;
+ * (lv_xattn/flash_attn_kernels.py:364-640, 677-819; launcher :904-1020, incl.
+ * the fp32 dQ scratch and `dq.copy_` of :1020) and the host-side
+ * `dk += dk_delta; dv += dv_delta` of lv_xattn/attn.py:523-524.
+ *   dq     : bf16, rows of the window are OVERWRITTEN (windows of different
+ *            rounds are disjoint, so nothing has to be accumulated);
  *   dk, dv : at Hkv heads (the group sum is taken in registers);
  *            dkv_accumulate == 0: bf16 tensors, overwritten;
- *            dkv_accumulate == 1: fp32 tensors of the same indexing, added to.
+ *            dkv_accumulate == 1: fp32 tensors of the same indexing, added to;
+ *   workspace : lvx_bwd_workspace_bytes(shape, row_count) bytes, 16-byte
+ *            aligned; holds scale*dS (bf16) between the two kernels of the call.
  */
 int lvx_bwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
             const lvx_tensor* v, const lvx_tensor* dout, const float* lse, const float* delta,
-            float* dq_acc, const lvx_tensor* dk, const lvx_tensor* dv, int32_t dkv_accumulate,
-            int32_t row_begin, int32_t row_count, void* stream);
+            const lvx_tensor* dq, const lvx_tensor* dk, const lvx_tensor* dv, int32_t dkv_accumulate,
+            int32_t row_begin, int32_t row_count, void* workspace, size_t workspace_bytes, void* stream);
+
+size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* shape, int32_t row_count);
 
 /*
  * dst(bf16, strided) = src(fp32, [B, H, L, D] contiguous): the final rounding of

@@ -51,6 +51,8 @@ constexpr int MAX_SPLITS = 16;
 
 }  // namespace
 
+static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch);
+
 extern "C" {
 
 int lvx_version(void) { return LVX_VERSION; }
@@ -197,27 +199,42 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
     return static_cast<int>(launch_preprocess(p, static_cast<hipStream_t>(stream)));
 }
 
+size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
+    if (!s || row_count <= 0) return 0;
+    const size_t tokens = ((size_t)s->Lkv + 127) / 128 * 128;
+    const size_t rows = ((size_t)row_count + 31) / 32 * 32;
+    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t);
+}
+
 int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
-            const lvx_tensor* dout, const float* lse, const float* delta, float* dq_acc,
+            const lvx_tensor* dout, const float* lse, const float* delta, const lvx_tensor* dq,
             const lvx_tensor* dk, const lvx_tensor* dv, int32_t dkv_accumulate,
-            int32_t row_begin, int32_t row_count, void* stream) {
+            int32_t row_begin, int32_t row_count, void* workspace, size_t workspace_bytes, void* stream) {
     LVX_TRY(check_shape(s));
     LVX_TRY(check_tensor(q));
     LVX_TRY(check_tensor(k));
     LVX_TRY(check_tensor(v));
     LVX_TRY(check_tensor(dout));
+    LVX_TRY(check_tensor(dq));
     LVX_TRY(check_tensor(dk));
     LVX_TRY(check_tensor(dv));
-    if (!lse || !delta || !dq_acc) return LVX_ERR_NULL;
-    if (!aligned16(dq_acc)) return LVX_ERR_ALIGN;
+    if (!lse || !delta) return LVX_ERR_NULL;
     if (dkv_accumulate != 0 && dkv_accumulate != 1) return LVX_ERR_SHAPE;
     LVX_TRY(check_rows(s, row_begin, row_count));
+    if (row_count == 0) return LVX_OK;
+    // row offsets inside a tensor are formed in 32 bits
+    if ((int64_t)s->Lq * q->stride_s >= (int64_t)1 << 31 || (int64_t)s->Lq * dout->stride_s >= (int64_t)1 << 31)
+        return LVX_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < lvx_bwd_workspace_bytes(s, row_count)) return LVX_ERR_WORKSPACE;
+    if (!aligned16(workspace)) return LVX_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
     BwdParams p{};
     p.q = static_cast<const uint16_t*>(q->ptr);
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
     p.dout = static_cast<const uint16_t*>(dout->ptr);
-    p.lse = lse; p.delta = delta; p.dq_acc = dq_acc;
+    p.lse = lse; p.delta = delta;
     p.dk = dk->ptr; p.dv = dv->ptr;
     p.qs = st3(q); p.ks = st3(k); p.vs = st3(v); p.dos = st3(dout); p.dks = st3(dk); p.dvs = st3(dv);
     p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
@@ -227,7 +244,31 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.total_wg = s->B * s->Hkv * p.n_kv_blocks;
     p.dkv_accumulate = dkv_accumulate;
     p.scale = s->scale; p.scale_log2e = s->scale * LOG2E;
-    return static_cast<int>(launch_bwd(p, s->kv_start != nullptr, static_cast<hipStream_t>(stream)));
+    const int64_t tokens = (int64_t)p.n_kv_blocks * 128;
+    const int64_t rows = ((int64_t)row_count + 31) / 32 * 32;
+    p.ds_ws = static_cast<uint16_t*>(workspace);
+    p.ws_ld = rows;
+    p.ws_bh = tokens * rows;
+    hipError_t e = launch_bwd(p, s->kv_start != nullptr, st);
+    if (e != hipSuccess) return static_cast<int>(e);
+
+    // dQ[b, h, rows, :] = dS^T[b, h]^T (rows x tokens) * K[b, h / G] (tokens x D), scale already in dS
+    GemmParams g{};
+    GemmProblem& pr = g.prob[0];
+    pr.A[0] = p.ds_ws; pr.lda[0] = rows;
+    pr.Bm[0] = p.k; pr.ldb[0] = k->stride_s;
+    pr.K[0] = s->Lkv; pr.nseg = 1;
+    pr.C = static_cast<uint16_t*>(dq->ptr) + (int64_t)row_begin * dq->stride_s;
+    pr.ldc = dq->stride_s;
+    g.M_ld = (int)rows;
+    g.batch_inner = s->Hq;
+    g.b_group = p.G;
+    g.a_batch = p.ws_bh;
+    g.b_outer = k->stride_b; g.b_inner = k->stride_h;
+    g.c_outer = dq->stride_b; g.c_inner = dq->stride_h;
+    g.k_len = s->kv_len;
+    fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
+    return static_cast<int>(launch_gemm(g, true, true, st));
 }
 
 int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L, int32_t D,
@@ -252,12 +293,20 @@ static int check_gemm_ptr(const void* p, int64_t ld) {
     return LVX_OK;
 }
 
-static void fill_grid(GemmParams& g, int M, int N, int nprob) {
+}  // extern "C"
+
+static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch = 1) {
     g.M = M; g.N = N; g.nprob = nprob;
+    if (g.M_ld < M) g.M_ld = M;
+    g.nbatch = nbatch;
+    if (g.batch_inner < 1) g.batch_inner = 1;
+    if (g.b_group < 1) g.b_group = 1;
     g.tiles_m = (M + 127) / 128;
     g.tiles_n = (N + 127) / 128;
-    g.total_wg = nprob * g.tiles_m * g.tiles_n;
+    g.total_wg = nprob * nbatch * g.tiles_m * g.tiles_n;
 }
+
+extern "C" {
 
 int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
                 void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, void* stream) {

@@ -71,8 +71,16 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
     const int tn = wid % p.tiles_n;
     const int t1 = wid / p.tiles_n;
     const int tm = t1 % p.tiles_m;
-    const GemmProblem& pr = p.prob[t1 / p.tiles_m];
+    const int t2 = t1 / p.tiles_m;
+    const int z = t2 % p.nbatch;
+    const GemmProblem& pr = p.prob[t2 / p.nbatch];
     const int m0 = tm * TM, n0 = tn * TN;
+    const int zo = z / p.batch_inner, zi = z % p.batch_inner;
+    const int64_t a_off = (int64_t)z * p.a_batch;
+    const int64_t b_off = zo * p.b_outer + (zi / p.b_group) * p.b_inner;
+    uint16_t* const Cz = pr.C + zo * p.c_outer + zi * p.c_inner;
+    int klen0 = pr.K[0];
+    if (p.k_len) klen0 = min(klen0, p.k_len[zo]);
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-    const int steps0 = (pr.K[0] + BK - 1) / BK;
+    const int steps0 = (klen0 + BK - 1) / BK;
     const int steps1 = pr.nseg > 1 ? (pr.K[1] + BK - 1) / BK : 0;
     const int steps = steps0 + steps1;
 
@@ -95,8 +103,9 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
     auto prefetch = [&](int s) {
         const int seg = s >= steps0 ? 1 : 0;
         const int k0 = (seg ? s - steps0 : s) * BK;
-        tile_load<A_MCONTIG>(apre, pr.A[seg], pr.lda[seg], m0, k0, p.M, pr.K[seg], tid);
-        tile_load<B_NCONTIG>(bpre, pr.Bm[seg], pr.ldb[seg], n0, k0, p.N, pr.K[seg], tid);
+        const int kl = seg ? pr.K[1] : klen0;
+        tile_load<A_MCONTIG>(apre, pr.A[seg] + a_off, pr.lda[seg], m0, k0, p.M_ld, kl, tid);
+        tile_load<B_NCONTIG>(bpre, pr.Bm[seg] + b_off, pr.ldb[seg], n0, k0, p.N, kl, tid);
     };
     if (steps > 0) prefetch(0);
 
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
                     u32x2 w;
                     w[0] = pack_bf16(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
                     w[1] = pack_bf16(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
-                    *reinterpret_cast<u32x2*>(pr.C + (int64_t)m * pr.ldc + n) = w;
+                    *reinterpret_cast<u32x2*>(Cz + (int64_t)m * pr.ldc + n) = w;
                 }
             }
     }

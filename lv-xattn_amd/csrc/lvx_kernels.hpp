@@ -61,7 +61,9 @@ struct BwdParams {
     const uint16_t* dout;
     const float* lse;
     const float* delta;
-    float* dq_acc;
+    uint16_t* ds_ws;           // dS^T workspace [B*Hq][tokens padded to 128][ws_ld]
+    int64_t ws_ld;             // elements per token row (row window padded to 32)
+    int64_t ws_bh;             // elements per (b, h) slab
     void* dk;
     void* dv;
     Strides3 qs, ks, vs, dos, dks, dvs;
@@ -93,11 +95,20 @@ struct GemmProblem {
     int64_t ldc;
 };
 
+// `nprob` problems of one shape, each repeated over `nbatch` batch entries.
+// Batch entry z = zo * batch_inner + zi addresses
+//   A + z * a_batch,  B + zo * b_outer + (zi / b_group) * b_inner,
+//   C + zo * c_outer + zi * c_inner
+// and, when k_len is given, contracts over only the first k_len[zo] values of k.
 struct GemmParams {
     GemmProblem prob[2];
     int nprob;
     int M, N;
+    int M_ld;                  // rows of A that may be loaded (>= M; rows in [M, M_ld) are padding)
     int tiles_m, tiles_n, total_wg;
+    int nbatch, batch_inner, b_group;
+    int64_t a_batch, b_outer, b_inner, c_outer, c_inner;
+    const int32_t* k_len;
 };
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st);

@@ -44,7 +44,9 @@ SYMBOLS = {
     "lvx_fwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, C.c_int32, C.c_int32, C.c_int32, _P, C.c_size_t, _P]),
     "lvx_merge": (C.c_int, [_SHAPE, _T, _P, _T, _P, C.c_int32, C.c_int32, _P]),
     "lvx_bwd_preprocess": (C.c_int, [_SHAPE, _T, _T, _P, C.c_int32, C.c_int32, _P]),
-    "lvx_bwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, _P, _P, _T, _T, C.c_int32, C.c_int32, C.c_int32, _P]),
+    "lvx_bwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, _P, _T, _T, _T, C.c_int32, C.c_int32, C.c_int32,
+                          _P, C.c_size_t, _P]),
+    "lvx_bwd_workspace_bytes": (C.c_size_t, [_SHAPE, C.c_int32]),
     "lvx_cast_f32_bf16": (C.c_int, [_P, _T, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_kv_proj": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, _P, C.c_int64,
                               C.c_int32, C.c_int32, C.c_int32, _P]),

@@ -109,8 +109,9 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     dk, dv [B,Hkv,Lkv,D]-shaped views of [B,Lkv,Hkv,D] memory, at the Hkv heads
     k and v came in with.  `o` and `L` are the finally merged forward results;
     every round uses them, so per-round contributions simply add
-    (attn.py:465-468, 509-527).  dQ, dK, dV are summed in fp32 across q heads of
-    a group and across rounds and rounded to bf16 once.
+    (attn.py:465-468, 509-527).  dK, dV are summed in fp32 across the q heads of
+    a group and across rounds and rounded to bf16 once; a round's dQ rows are
+    complete after that round (fp32 sum over all local tokens, rounded once).
     `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored."""
     _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
     q_, k_, v_, o_, do_ = (_usable(t) for t in (q, k, v, o, do))
@@ -123,17 +124,18 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     L_ = L.to(torch.float32).reshape(B * Hq, Lq).contiguous()
 
     delta = workspace("bwd_delta", (B * Hq, Lq), torch.float32, dev)
-    dq_acc = workspace("bwd_dq_acc", (B, Hq, Lq, D), torch.float32, dev)
-    dq_acc.zero_()
     dq = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
     dk = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
     dv = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
+    ws = workspace("bwd_ds", (ops.bwd_workspace_bytes(q_, k_, max(r1 - r0 for r0, r1 in windows)),),
+                   torch.uint8, dev)
     if len(windows) == 1:
         r0, r1 = windows[0]
         ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
-        ops.bwd(q_, k_, v_, do_, L_, delta, dq_acc, dk, dv, sm_scale, r0, r1 - r0, mask, accumulate_dkv=False)
+        ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk, dv, sm_scale, r0, r1 - r0, mask, accumulate_dkv=False,
+                workspace=ws)
     else:
         dk_acc = workspace("bwd_dk_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
         dv_acc = workspace("bwd_dv_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
@@ -141,10 +143,9 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
         dv_acc.zero_()
         for r0, r1 in windows:
             ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
-            ops.bwd(q_, k_, v_, do_, L_, delta, dq_acc, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
-                    accumulate_dkv=True)
+            ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
+                    accumulate_dkv=True, workspace=ws)
         # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
         ops.cast_f32_bf16(dk_acc.transpose(1, 2), dk.transpose(1, 2))
         ops.cast_f32_bf16(dv_acc.transpose(1, 2), dv.transpose(1, 2))
-    ops.cast_f32_bf16(dq_acc, dq)
     return dq, dk, dv

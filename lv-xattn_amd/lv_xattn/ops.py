@@ -96,23 +96,33 @@ def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
     check(rc, "lvx_bwd_preprocess")
 
 
-def bwd(q, k, v, dout, lse, delta, dq_acc, dk, dv, scale, row_begin=0, row_count=None,
-        mask: Optional[Mask] = None, accumulate_dkv: bool = False) -> None:
-    """Adds the selected rows' contribution to dq_acc (fp32 [B,Hq,Lq,D]) and
-    writes (bf16) or accumulates (fp32) dk, dv at Hkv heads."""
+def bwd_workspace_bytes(q, k, row_count: int) -> int:
+    s = _shape(q, k, 1.0, None)
+    return int(load().lvx_bwd_workspace_bytes(C.byref(s), row_count))
+
+
+def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=None,
+        mask: Optional[Mask] = None, accumulate_dkv: bool = False,
+        workspace: Optional[torch.Tensor] = None) -> None:
+    """Writes dq (bf16) for the selected rows and writes (bf16) or accumulates
+    (fp32) dk, dv at Hkv heads.  `workspace`: uint8 tensor of at least
+    bwd_workspace_bytes(q, k, row_count) bytes."""
     s = _shape(q, k, scale, mask)
     if row_count is None:
         row_count = q.shape[2] - row_begin
     _check_lse(lse, q)
     _check_lse(delta, q)
-    if dq_acc.dtype != torch.float32 or not dq_acc.is_contiguous() or dq_acc.shape != q.shape:
-        raise LvxError("dq_acc must be a contiguous fp32 tensor shaped like q")
+    if dq.dtype != torch.bfloat16 or dq.shape != q.shape:
+        raise LvxError("dq must be a bf16 tensor shaped like q")
     want = torch.float32 if accumulate_dkv else torch.bfloat16
     if dk.dtype != want or dv.dtype != want or dk.shape != k.shape or dv.shape != k.shape:
         raise LvxError(f"dk/dv must be {want} tensors shaped like k")
+    if workspace is None:
+        workspace = torch.empty(bwd_workspace_bytes(q, k, row_count), dtype=torch.uint8, device=q.device)
     rc = load().lvx_bwd(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(dout)),
-                        lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr(), C.byref(t4(dk)), C.byref(t4(dv)),
-                        1 if accumulate_dkv else 0, row_begin, row_count, stream_ptr())
+                        lse.data_ptr(), delta.data_ptr(), C.byref(t4(dq)), C.byref(t4(dk)), C.byref(t4(dv)),
+                        1 if accumulate_dkv else 0, row_begin, row_count,
+                        workspace.data_ptr(), workspace.numel() * workspace.element_size(), stream_ptr())
     check(rc, "lvx_bwd")
 
 

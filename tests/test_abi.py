@@ -92,10 +92,16 @@ def test_other_entry_points_reject_bad_arguments(lib):
     assert lib.lvx_merge(C.byref(s), C.byref(t), None, C.byref(t), 0x2000, 0, 64, None) == -1
     assert lib.lvx_merge(C.byref(s), C.byref(t), 0x2000, C.byref(t), 0x2000, 0, 65, None) == -3
     assert lib.lvx_bwd_preprocess(C.byref(s), C.byref(t), C.byref(_t(ptr=8)), 0x2000, 0, 64, None) == -2
-    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, None,
-                       C.byref(t), C.byref(t), 0, 0, 64, None) == -1
-    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, 0x3000,
-                       C.byref(t), C.byref(t), 2, 0, 64, None) == -3
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, None, C.byref(t),
+                       C.byref(t), C.byref(t), 0, 0, 64, 0x4000, 1 << 30, None) == -1
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
+                       C.byref(t), C.byref(t), 2, 0, 64, 0x4000, 1 << 30, None) == -3
+    need = lib.lvx_bwd_workspace_bytes(C.byref(s), 64)
+    assert need == 8 * 256 * 64 * 2
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
+                       C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need - 1, None) == -7
+    assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
+                       C.byref(t), C.byref(t), 0, 0, 64, None, 0, None) == -7
     assert lib.lvx_cast_f32_bf16(0x1000, C.byref(t), 1, 8, 64, 64, None) == -4
     assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, None) == -3
     assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, None) == -1
