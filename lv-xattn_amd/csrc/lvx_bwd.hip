@@ -42,10 +42,16 @@ namespace {
 constexpr int D = 128;
 constexpr int BN = 128;       // visual tokens per work-group
 constexpr int BM = 32;        // text rows per step
-constexpr int QS = D + 8;     // row stride of the Q / dO tiles (68 dwords: 16-byte row reads conflict-free)
+// Every Q / dO tile is staged twice, because no single row stride serves both
+// access patterns without bank conflicts: 16-byte row reads want 16 consecutive
+// rows on 16 distinct bank quads (68-dword rows), a transposing read touches 8
+// rows x 16 dwords and wants them to tile the 64 banks twice (72-dword rows).
+constexpr int QS = D + 8;     // row stride of the copy read by rows      (stage 1)
+constexpr int QT = D + 16;    // row stride of the copy read transposed   (stage 3)
 constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row] (80 bytes, 16-byte aligned rows)
 
-constexpr int QD_ELEMS = 2 * BM * QS;          // one (Q, dO) tile pair
+constexpr int QD_ELEMS = 2 * BM * QS + 2 * BM * QT;   // one (Q, dO) tile pair, both copies
+constexpr int OFF_T = 2 * BM * QS;                   // transposed-read copies inside a pair
 constexpr int DST_ELEMS = BN * DSS;            // one dS^T tile
 constexpr int OFF_QD = 0;
 constexpr int OFF_DST = OFF_QD + 3 * QD_ELEMS;
@@ -103,6 +109,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     const int s_chunk = st & 15, s_group = st >> 4;
     const bool is_do = tid >= 128;
     const int stage_off = (is_do ? BM * QS : 0) + 4 * s_group * QS + s_chunk * 8;
+    const int stage_off_t = OFF_T + (is_do ? BM * QT : 0) + 4 * s_group * QT + s_chunk * 8;
     const uint16_t* g_base = is_do ? p.dout + b * p.dos.b : p.q + b * p.qs.b;
     const int64_t g_hs = is_do ? p.dos.h : p.qs.h;
     const int g_rs = (int)(is_do ? p.dos.s : p.qs.s);
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     }
 
     // per-lane offset of the transposing operand reads (Q^T / dO^T, rows in accumulator order)
-    const int off_qT = tr_lane_offset(lane, QS, true);
+    const int off_qT = OFF_T + tr_lane_offset(lane, QT, true);
     // dS^T copy-out: 512 chunks of 16 bytes per tile, two per thread
     const int cp_token = tid >> 2, cp_part = tid & 3;
     uint16_t* ws_lane = p.ds_ws + ((int64_t)kvb + cp_token) * p.ws_ld + cp_part * 8;
@@ -160,7 +167,10 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 
     auto stage_write = [&](uint16_t* qd, u32x4* meta) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(qd + stage_off + i * QS) = pre[i];
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<u32x4*>(qd + stage_off + i * QS) = pre[i];
+            *reinterpret_cast<u32x4*>(qd + stage_off_t + i * QT) = pre[i];
+        }
         const float l = __uint_as_float(pre_m);
         // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
         const float lt = (!pre_ok || l == -INFINITY) ? INFINITY : l * LOG2E;
@@ -246,8 +256,8 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16x8 a1 = lds_operand_tr(qt + BM * QS + 16 * j * QS + dt * 32, 8 * QS);
-                const bf16x8 a2 = lds_operand_tr(qt + 16 * j * QS + dt * 32, 8 * QS);
+                const bf16x8 a1 = lds_operand_tr(qt + BM * QT + 16 * j * QT + dt * 32, 8 * QT);
+                const bf16x8 a2 = lds_operand_tr(qt + 16 * j * QT + dt * 32, 8 * QT);
                 dv[dt] = mfma32(a1, pb[j], dv[dt]);
                 dk[dt] = mfma32(a2, dsb[j], dk[dt]);
             }
@@ -259,6 +269,9 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const u32x4 w = *reinterpret_cast<const u32x4*>(dst + (cp_token + 64 * j) * DSS + cp_part * 8);
+#ifdef LVX_EXP_NOSTORE
+            if (w[0] == 0x12345678u)
+#endif
             *reinterpret_cast<u32x4*>(gp + (int64_t)64 * j * p.ws_ld) = w;
         }
     };
