@@ -247,7 +247,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     const int64_t tokens = (int64_t)p.n_kv_blocks * 128;
     const int64_t rows = ((int64_t)row_count + 31) / 32 * 32;
     p.ds_ws = static_cast<uint16_t*>(workspace);
-    p.ws_ld = rows;
+    p.ws_ld = rows * 128;          // one token block: (rows / 32) tiles of 128 x 32
     p.ws_bh = tokens * rows;
     hipError_t e = launch_bwd(p, s->kv_start != nullptr, st);
     if (e != hipSuccess) return static_cast<int>(e);
@@ -267,6 +267,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.b_outer = k->stride_b; g.b_inner = k->stride_h;
     g.c_outer = dq->stride_b; g.c_inner = dq->stride_h;
     g.k_len = s->kv_len;
+    g.a_tiled_m = (int)(rows / 32);
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
     return static_cast<int>(launch_gemm(g, true, true, st));
 }

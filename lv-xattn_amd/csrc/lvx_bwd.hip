@@ -2,34 +2,34 @@
 //   P = exp(scale*Q K^T - LSE);  dV = P^T dO;  dP = dO V^T;
 //   dS = P * (dP - delta);  dK = scale * dS^T Q;  dQ = scale * dS K.
 //
-// Mapping.  A work-group (4 waves, one per SIMD) owns a block of 128 visual
-// tokens of one kv head and streams every text row of the window for every q
-// head of the GQA group past it, 32 rows at a time.  Wave w owns tokens
-// 32w..32w+31 of the block: its K and V rows sit in registers as MFMA B
-// operands for the whole kernel, and its dK^T / dV^T (128 x 32 each, fp32) stay
-// in accumulators until the end, so the sum over the q heads of the group and
-// over all rows never leaves the register file.
+// Mapping.  A work-group owns a block of 128 visual tokens of one kv head and
+// streams every text row of the window for every q head of the GQA group past
+// it, 32 rows at a time.  It has 8 waves, two per SIMD, in two roles; waves w
+// and w+4 share token slice 32w..32w+31 of the block:
+//   P-wave  (w)   : S = Q K^T, P = exp2(..), dV^T += dO^T P     K rows + dV^T resident
+//   D-wave  (w+4) : dP = dO V^T, dS = P (dP - delta) scale,
+//                   dK^T += Q^T dS                              V rows + dK^T resident
+// so each wave keeps 64 accumulator registers and 32 operand registers for the
+// whole kernel (the sum over the q heads of the group and over all rows never
+// leaves the register file) and fits two to a SIMD: while one wave waits for
+// LDS or runs its exp2/multiplies, the other feeds the MFMA pipe.  P travels
+// from the P-wave to the D-wave as bf16 through LDS (32 bytes per lane), one
+// step behind, so the one barrier per step also orders that hand-over.
 //
 // dQ = scale * dS K sums over ALL tokens, i.e. over every work-group of the kv
 // head.  Adding 51 partial tiles per row with fp32 atomics costs more than the
 // whole rest of the kernel on this machine (atomic adds sustain about 1.3 TB/s),
-// so dQ is not formed here: the waves gather scale*dS (bf16) in LDS and stream
-// it to a workspace dS^T[b, h, token, row] in HBM with full 64-byte segments,
-// and a batched GEMM (launched by the caller right after) contracts it with K.
-// The workspace costs 2 bytes per (row, token, head) written once and read once.
+// so dQ is not formed here: the D-waves gather scale*dS (bf16) in LDS and the
+// group streams it to a workspace in HBM, one contiguous 8 KB tile
+// [128 tokens][32 rows] per step, indexed [b, h, token block, row tile]; a
+// batched GEMM (launched by the caller right after) contracts it with K.  The workspace costs 2 bytes per (row, token, head),
+// written once and read once.
 //
-// Per 32-row step and wave (all MFMA are 32x32x16 bf16):
-//   (1) S, dP        2 x 8 MFMA   A = Q / dO rows from LDS (16-byte reads)
-//   (2) P, dS        VALU only    exp2, the two multiplies, bf16 packing
-//   (3) dV^T, dK^T   2 x 8 MFMA   A = dO^T / Q^T, read from the SAME row-major
-//                                 LDS tiles with the transposing LDS read; B =
-//                                 P / dS straight from the registers of (2)
-//   (4) dS^T store   LDS -> HBM   the [128 tokens][32 rows] tile the waves wrote
-// With one wave per SIMD nothing else hides the VALU work of (2), so the loop is
-// software-pipelined: the body of step i runs (1) and (2) of tile i together
-// with (3) and (4) of tile i-1, which are independent of them.  Q/dO tiles are
-// triple-buffered in LDS and the dS^T tile and row metadata double-buffered, so
-// one barrier per step is enough.
+// All MFMA are 32x32x16 bf16.  A operands come from LDS: Q / dO rows by 16-byte
+// reads, Q^T / dO^T by the transposing LDS read of a second copy of the same
+// row-major tile (no single row stride is conflict-free for both patterns), the
+// latter addressed in the accumulator's row order so that P / dS go from the
+// registers straight into the next MFMA as B operands.
 #include <type_traits>
 
 #include "lvx_common.hpp"
@@ -42,29 +42,32 @@ namespace {
 constexpr int D = 128;
 constexpr int BN = 128;       // visual tokens per work-group
 constexpr int BM = 32;        // text rows per step
-// Every Q / dO tile is staged twice, because no single row stride serves both
-// access patterns without bank conflicts: 16-byte row reads want 16 consecutive
-// rows on 16 distinct bank quads (68-dword rows), a transposing read touches 8
-// rows x 16 dwords and wants them to tile the 64 banks twice (72-dword rows).
-constexpr int QS = D + 8;     // row stride of the copy read by rows      (stage 1)
-constexpr int QT = D + 16;    // row stride of the copy read transposed   (stage 3)
-constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row] (80 bytes, 16-byte aligned rows)
+constexpr int NT = 512;       // threads per work-group
+constexpr int QS = D + 8;     // row stride of the tile copies read by rows       (68 dwords)
+constexpr int QT = D + 16;    // row stride of the tile copies read transposed    (72 dwords)
+constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row]
 
-constexpr int QD_ELEMS = 2 * BM * QS + 2 * BM * QT;   // one (Q, dO) tile pair, both copies
-constexpr int OFF_T = 2 * BM * QS;                   // transposed-read copies inside a pair
-constexpr int DST_ELEMS = BN * DSS;            // one dS^T tile
-constexpr int OFF_QD = 0;
-constexpr int OFF_DST = OFF_QD + 3 * QD_ELEMS;
-constexpr int SMEM_ELEMS = OFF_DST + 2 * DST_ELEMS;
+// one staged (Q, dO) tile set: Q rows | dO rows | Q for transposed reads | dO for transposed reads
+constexpr int OFF_QR = 0;
+constexpr int OFF_DOR = OFF_QR + BM * QS;
+constexpr int OFF_QTR = OFF_DOR + BM * QS;
+constexpr int OFF_DOTR = OFF_QTR + BM * QT;
+constexpr int QD_ELEMS = OFF_DOTR + BM * QT;
+constexpr int DST_ELEMS = BN * DSS;
+constexpr int PB_ELEMS = 4 * 2 * 64 * 8;       // P hand-over: [slice][half][lane][16 bytes] as uint16
+constexpr int OFF_QD = 0;                      // x3
+constexpr int OFF_DST = OFF_QD + 3 * QD_ELEMS; // x2
+constexpr int OFF_PB = OFF_DST + 2 * DST_ELEMS;  // x2
+constexpr int SMEM_ELEMS = OFF_PB + 2 * PB_ELEMS;
 
 constexpr float LOG2E = 1.4426950408889634f;
 
 template <bool MASKED>
-__global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     __shared__ __attribute__((aligned(16))) uint16_t smem[SMEM_ELEMS];
-    // per-row metadata of a staged tile, double-buffered: 8 x 16 bytes each of
+    // per-row metadata of a staged tile, triple-buffered: 8 x 16 bytes each of
     // LSE*log2e, delta, kv_start, kv_end
-    __shared__ u32x4 meta_s4[2][BM];
+    __shared__ u32x4 meta_s4[3][BM];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
@@ -74,46 +77,48 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     const int b = bh / p.Hkv;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int slice = wave & 3;
+    const bool d_role = wave >= 4;
 
     int kv_len = p.Lkv;
     if (p.kv_len) kv_len = min(p.kv_len[b], p.Lkv);
     const int kvb = kblk * BN;
-    const int my_kv = kvb + 32 * wave + l32;
+    const int my_kv = kvb + 32 * slice + l32;
     const bool kv_valid = my_kv < kv_len;
     const bool tail_block = kvb + BN > kv_len;
 
-    const uint16_t* kbase = p.k + b * p.ks.b + hk * p.ks.h;
-    const uint16_t* vbase = p.v + b * p.vs.b + hk * p.vs.h;
-
-    // ---- prologue: K, V rows of this wave as B operands (contraction over d)
-    bf16x8 kreg[8], vreg[8];
+    // ---- resident B operand: this wave's K rows (P-wave) or V rows (D-wave)
+    bf16x8 breg[8];
+    {
+        const uint16_t* base = d_role ? p.v + b * p.vs.b + hk * p.vs.h + (int64_t)my_kv * p.vs.s
+                                      : p.k + b * p.ks.b + hk * p.ks.h + (int64_t)my_kv * p.ks.s;
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-        kreg[kk] = as_bf16x8(ldg16(kbase + (int64_t)my_kv * p.ks.s + kk * 16 + g * 8, kv_valid));
-        vreg[kk] = as_bf16x8(ldg16(vbase + (int64_t)my_kv * p.vs.s + kk * 16 + g * 8, kv_valid));
+        for (int kk = 0; kk < 8; ++kk) breg[kk] = as_bf16x8(ldg16(base + kk * 16 + g * 8, kv_valid));
     }
-
-    f32x16 dk[4], dv[4];
+    // ---- resident accumulator: dV^T (P-wave) or dK^T (D-wave), [128 d][32 tokens]
+    f32x16 acc[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { dk[dt][v] = 0.f; dv[dt][v] = 0.f; }
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
 
     const int n_qtiles = (p.row_end - p.row_begin + BM - 1) / BM;
     const int n_iter = (kvb < kv_len) ? p.G * n_qtiles : 0;
     const float c = p.scale_log2e;
 
-    // staging role of this thread: threads 0..127 carry Q, 128..255 carry dO
-    const int st = tid & 127;
-    const int s_chunk = st & 15, s_group = st >> 4;
-    const bool is_do = tid >= 128;
-    const int stage_off = (is_do ? BM * QS : 0) + 4 * s_group * QS + s_chunk * 8;
-    const int stage_off_t = OFF_T + (is_do ? BM * QT : 0) + 4 * s_group * QT + s_chunk * 8;
+    // staging role of this thread: threads 0..255 carry Q, 256..511 carry dO; two
+    // 16-byte chunks each (rows s_row and s_row + 16)
+    const int st = tid & 255;
+    const int s_row = st >> 4, s_chunk = st & 15;
+    const bool is_do = tid >= 256;
+    const int stage_off = (is_do ? OFF_DOR : OFF_QR) + s_row * QS + s_chunk * 8;
+    const int stage_off_t = (is_do ? OFF_DOTR : OFF_QTR) + s_row * QT + s_chunk * 8;
     const uint16_t* g_base = is_do ? p.dout + b * p.dos.b : p.q + b * p.qs.b;
     const int64_t g_hs = is_do ? p.dos.h : p.qs.h;
     const int g_rs = (int)(is_do ? p.dos.s : p.qs.s);
-    const int meta_kind = (tid >> 5) & 3;    // 0 LSE, 1 delta, 2 kv_start, 3 kv_end
+    const int meta_kind = (tid >> 5) & 3;    // 0 LSE, 1 delta, 2 kv_start, 3 kv_end (threads 0..127)
     const uint32_t* m_base = reinterpret_cast<const uint32_t*>(p.lse);
     int64_t m_hs = p.Lq;
     if (meta_kind == 1) m_base = reinterpret_cast<const uint32_t*>(p.delta);
@@ -124,11 +129,13 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
         m_base += (int64_t)b * p.Hq * p.Lq;
     }
 
-    // per-lane offset of the transposing operand reads (Q^T / dO^T, rows in accumulator order)
-    const int off_qT = OFF_T + tr_lane_offset(lane, QT, true);
-    // dS^T copy-out: 512 chunks of 16 bytes per tile, two per thread
+    // per-lane offsets: transposing operand reads (rows in accumulator order),
+    // P hand-over slot, dS^T copy-out (512 chunks of 16 bytes, one per thread)
+    const int off_tr = tr_lane_offset(lane, QT, true);
+    const int pb_off = slice * (2 * 64 * 8) + lane * 8;
     const int cp_token = tid >> 2, cp_part = tid & 3;
-    uint16_t* ws_lane = p.ds_ws + ((int64_t)kvb + cp_token) * p.ws_ld + cp_part * 8;
+    // workspace tile (b, h, token block, row tile): [128 tokens][32 rows], 8 KB, contiguous
+    uint16_t* ws_lane = p.ds_ws + (int64_t)kblk * p.ws_ld + cp_token * BM + cp_part * 8;
 
     // token blocks of one kv head walk the (head, row tile) list from different
     // starting points, which spreads their reads of Q / dO over the L2
@@ -142,21 +149,32 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
     // Every load is unconditional: rows past the window are clamped to its last
     // row (their LSE is forced to +inf, so P = 0 and nothing they carry reaches a
     // result), and the fetch after the last tile re-reads some tile.
-    u32x4 pre[4];
-    uint32_t pre_m = 0;
-    bool pre_ok = false;
-    auto prefetch = [&]() {
+    // Two register sets alternate: the set consumed at the top of step i is
+    // refilled right after the barrier with tile i + 2, so every load has two
+    // full steps to arrive.
+    struct Pre {
+        u32x4 d[2];
+        uint32_t m;
+        bool ok;
+    };
+    Pre preA{}, preB{};
+    int exp_loads = 0;
+    auto prefetch = [&](Pre& pr) {
+#ifdef LVX_EXP_NOLOAD
+        if (exp_loads >= 2) return;
+        ++exp_loads;
+#endif
         const int h = hk * p.G + cur_gi;
         const int r0 = p.row_begin + cur_qt * BM;
         const uint16_t* base = g_base + h * g_hs + s_chunk * 8;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = min(r0 + 4 * s_group + i, p.row_end - 1);
-            pre[i] = *reinterpret_cast<const u32x4*>(base + row * g_rs);
+        for (int i = 0; i < 2; ++i) {
+            const int row = min(r0 + s_row + 16 * i, p.row_end - 1);
+            pr.d[i] = *reinterpret_cast<const u32x4*>(base + row * g_rs);
         }
         const int mrow = r0 + (tid & 31);
-        pre_ok = mrow < p.row_end;
-        pre_m = m_base[h * m_hs + min(mrow, p.row_end - 1)];   // used one step later
+        pr.ok = mrow < p.row_end;
+        pr.m = m_base[h * m_hs + min(mrow, p.row_end - 1)];
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
         if (++cur_qt == n_qtiles) {
@@ -164,51 +182,45 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
             if (++cur_gi == p.G) cur_gi = 0;
         }
     };
-
-    auto stage_write = [&](uint16_t* qd, u32x4* meta) {
+    auto stage_write = [&](const Pre& pr, uint16_t* qd, u32x4* meta) {
+#ifdef LVX_EXP_NOSTAGE
+        if (pr.m == 0x12345678u)
+#endif
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4*>(qd + stage_off + i * QS) = pre[i];
-            *reinterpret_cast<u32x4*>(qd + stage_off_t + i * QT) = pre[i];
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<u32x4*>(qd + stage_off + 16 * i * QS) = pr.d[i];
+            *reinterpret_cast<u32x4*>(qd + stage_off_t + 16 * i * QT) = pr.d[i];
         }
-        const float l = __uint_as_float(pre_m);
+        const float l = __uint_as_float(pr.m);
         // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
-        const float lt = (!pre_ok || l == -INFINITY) ? INFINITY : l * LOG2E;
-        const uint32_t m = meta_kind == 0 ? __float_as_uint(lt) : (pre_ok ? pre_m : 0u);
-        reinterpret_cast<uint32_t*>(meta)[tid & 127] = m;   // both halves write the same words
+        const float lt = (!pr.ok || l == -INFINITY) ? INFINITY : l * LOG2E;
+        const uint32_t m = meta_kind == 0 ? __float_as_uint(lt) : (pr.ok ? pr.m : 0u);
+        reinterpret_cast<uint32_t*>(meta)[tid & 127] = m;   // the four quarters write the same words
     };
 
-    // (1) S = Q K_w^T, dP = dO V_w^T : rows = text rows, cols = this wave's tokens
-    auto stage1 = [&](const uint16_t* qd, f32x16& s, f32x16& dp) {
-        const uint16_t* qrow = qd + l32 * QS + g * 8;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-            const bf16x8 aq = *reinterpret_cast<const bf16x8*>(qrow + kk * 16);
-            const bf16x8 ad = *reinterpret_cast<const bf16x8*>(qrow + BM * QS + kk * 16);
-            s = mfma32(aq, kreg[kk], s);
-            dp = mfma32(ad, vreg[kk], dp);
-        }
+    // the finished dS^T tile goes to HBM as one contiguous 8 KB block
+    auto copy_out = [&](const uint16_t* dst, int h, int r0) {
+        uint16_t* gp = ws_lane + ((int64_t)b * p.Hq + h) * p.ws_bh + (int64_t)((r0 - p.row_begin) / BM) * (BN * BM);
+#ifndef LVX_EXP_NOSTORE
+        *reinterpret_cast<u32x4*>(gp) = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
+#endif
     };
 
-    // (2) P and scale*dS as bf16 B operands (register v of lane-half g is text
-    //     row 8*(v/4)+4g+(v%4)), and scale*dS handed to the other waves as
-    //     dST[token of the block][text row]
-    auto stage2 = [&](auto tail_c, f32x16& s, f32x16& dp, const u32x4* meta, uint16_t* dst, bf16x8 pb[2],
-                      bf16x8 dsb[2]) {
+    // ---- P-wave: S = Q K_w^T, P = exp2(S*c - LSE*log2e) (masked), hand P over, dV_w^T += dO^T P
+    auto p_step = [&](auto tail_c, const uint16_t* qd, const u32x4* meta, uint16_t* pbuf) {
         constexpr bool TAIL = decltype(tail_c)::value;
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+        const uint16_t* qrow = qd + OFF_QR + l32 * QS + g * 8;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            s = mfma32(*reinterpret_cast<const bf16x8*>(qrow + kk * 16), breg[kk], s);
 #pragma unroll
         for (int vg = 0; vg < 4; ++vg) {
             const f32x4 l4 = __builtin_bit_cast(f32x4, meta[2 * vg + g]);
-            const f32x4 d4 = __builtin_bit_cast(f32x4, meta[8 + 2 * vg + g]);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int v = 4 * vg + r;
-                const float pv = __builtin_amdgcn_exp2f(fmaf(s[v], c, -l4[r]));
-                s[v] = pv;
-                dp[v] = pv * p.scale * (dp[v] - d4[r]);
-            }
+            for (int r = 0; r < 4; ++r) s[4 * vg + r] = __builtin_amdgcn_exp2f(fmaf(s[4 * vg + r], c, -l4[r]));
         }
         if (MASKED) {
 #pragma unroll
@@ -219,151 +231,158 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
                 for (int r = 0; r < 4; ++r) {
                     const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
                     s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
-                    dp[4 * vg + r] = vis ? dp[4 * vg + r] : 0.f;
                 }
             }
         } else if (TAIL) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                s[v] = kv_valid ? s[v] : 0.f;
-                dp[v] = kv_valid ? dp[v] : 0.f;
-            }
+            for (int v = 0; v < 16; ++v) s[v] = kv_valid ? s[v] : 0.f;
         }
+        u32x4 pu[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pu[j][e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
+        *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
+        *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
+        const uint16_t* dot = qd + OFF_DOTR + off_tr;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[dt] = mfma32(lds_operand_tr(dot + 16 * j * QT + dt * 32, 8 * QT), as_bf16x8(pu[j]), acc[dt]);
+    };
+
+    // ---- D-wave, first half: dP = dO V_w^T of the current tile
+    auto d_step_dp = [&](const uint16_t* qd, f32x16& dp) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[v] = 0.f;
+        const uint16_t* drow = qd + OFF_DOR + l32 * QS + g * 8;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            dp = mfma32(*reinterpret_cast<const bf16x8*>(drow + kk * 16), breg[kk], dp);
+    };
+    // ---- D-wave, second half (one step later): dS = P (dP - delta) scale, dS^T to LDS, dK_w^T += Q^T dS
+    auto d_step_ds = [&](const uint16_t* qd, const u32x4* meta, const uint16_t* pbuf, uint16_t* dst,
+                         const f32x16& dp) {
+        u32x4 pu[2];
+        pu[0] = *reinterpret_cast<const u32x4*>(pbuf + pb_off);
+        pu[1] = *reinterpret_cast<const u32x4*>(pbuf + pb_off + 64 * 8);
         u32x4 dsu[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            u32x4 u;
+            const f32x4 da = __builtin_bit_cast(f32x4, meta[8 + 4 * j + g]);       // rows 16j + 4g + 0..3
+            const f32x4 db = __builtin_bit_cast(f32x4, meta[8 + 4 * j + 2 + g]);   // rows 16j + 8 + 4g + 0..3
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                u[e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
-                dsu[j][e] = pack_bf16(dp[8 * j + 2 * e], dp[8 * j + 2 * e + 1]);
+                // registers 8j + 2e, 8j + 2e + 1 are rows 16j + 8(e/2) + 4g + 2(e%2) + {0, 1}
+                const float d0 = (e < 2) ? da[2 * (e & 1)] : db[2 * (e & 1)];
+                const float d1 = (e < 2) ? da[2 * (e & 1) + 1] : db[2 * (e & 1) + 1];
+                const float p0 = bf16_lo(pu[j][e]) * p.scale, p1 = bf16_hi(pu[j][e]) * p.scale;
+                dsu[j][e] = pack_bf16(p0 * (dp[8 * j + 2 * e] - d0), p1 * (dp[8 * j + 2 * e + 1] - d1));
             }
-            pb[j] = as_bf16x8(u);
-            dsb[j] = as_bf16x8(dsu[j]);
         }
-        uint16_t* dsp = dst + (32 * wave + l32) * DSS + 4 * g;
+        uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
 #pragma unroll
         for (int vg = 0; vg < 4; ++vg) {
             const u32x2 w = {dsu[vg >> 1][2 * (vg & 1)], dsu[vg >> 1][2 * (vg & 1) + 1]};
             *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
         }
-    };
-
-    // (3) dV_w^T += dO^T P,  dK_w^T += Q^T (scale*dS)  (contraction over the 32 text rows)
-    auto stage3 = [&](const uint16_t* qd, const bf16x8 pb[2], const bf16x8 dsb[2]) {
-        const uint16_t* qt = qd + off_qT;
+        const uint16_t* qt = qd + OFF_QTR + off_tr;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const bf16x8 a1 = lds_operand_tr(qt + BM * QT + 16 * j * QT + dt * 32, 8 * QT);
-                const bf16x8 a2 = lds_operand_tr(qt + 16 * j * QT + dt * 32, 8 * QT);
-                dv[dt] = mfma32(a1, pb[j], dv[dt]);
-                dk[dt] = mfma32(a2, dsb[j], dk[dt]);
-            }
-    };
-
-    // (4) the finished dS^T tile goes to HBM: dS^T[b, h, token, row - row_begin]
-    auto stage4 = [&](const uint16_t* dst, int h, int r0) {
-        uint16_t* gp = ws_lane + ((int64_t)b * p.Hq + h) * p.ws_bh + (r0 - p.row_begin);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const u32x4 w = *reinterpret_cast<const u32x4*>(dst + (cp_token + 64 * j) * DSS + cp_part * 8);
-#ifdef LVX_EXP_NOSTORE
-            if (w[0] == 0x12345678u)
-#endif
-            *reinterpret_cast<u32x4*>(gp + (int64_t)64 * j * p.ws_ld) = w;
-        }
+            for (int j = 0; j < 2; ++j)
+                acc[dt] = mfma32(lds_operand_tr(qt + 16 * j * QT + dt * 32, 8 * QT), as_bf16x8(dsu[j]), acc[dt]);
     };
 
     auto run = [&](auto tail_c) {
         if (n_iter == 0) return;
-        uint16_t* qd0 = smem + OFF_QD;                 // tile being staged / used by (1),(2)
-        uint16_t* qd1 = smem + OFF_QD + QD_ELEMS;      // next to be staged
-        uint16_t* qd2 = smem + OFF_QD + 2 * QD_ELEMS;  // previous tile, used by (3)
-        uint16_t* ds0 = smem + OFF_DST;
-        uint16_t* ds1 = smem + OFF_DST + DST_ELEMS;
-        int mb = 0;
-
-        bf16x8 pb[2], dsb[2];
-        f32x16 s, dp;
-        int h_prev, r0_prev;          // tile whose (3), (4) run in the current step
-
-        // ---- first tile: (1), (2) only
-        prefetch();
-        h_prev = hk * p.G + cur_gi;
-        r0_prev = p.row_begin + cur_qt * BM;
-        advance();
-        stage_write(qd0, meta_s4[0]);
-        __syncthreads();
-        prefetch();
-        stage1(qd0, s, dp);
-        stage2(tail_c, s, dp, meta_s4[0], ds0, pb, dsb);
-
-        // ---- steady state: (1), (2) of tile i with (3), (4) of tile i-1
-        for (int i = 1; i < n_iter; ++i) {
-            { uint16_t* t = qd2; qd2 = qd0; qd0 = qd1; qd1 = t; }   // rotate tile buffers
-            { uint16_t* t = ds0; ds0 = ds1; ds1 = t; }              // ds1 = dS^T of tile i-1
-            mb ^= 1;
-            const int h_cur = hk * p.G + cur_gi;
-            const int r0_cur = p.row_begin + cur_qt * BM;
+        // tile i lives in qd(i % 3), meta_s4[i % 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
+        auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
+        auto dst = [&](int k) { return smem + OFF_DST + k * DST_ELEMS; };
+        auto pbf = [&](int k) { return smem + OFF_PB + k * PB_ELEMS; };
+        // (h, r0) of the tiles: being fetched (+2, +1), current (0), previous (-1, -2)
+        int h_q[5] = {0, 0, 0, 0, 0}, r_q[5] = {0, 0, 0, 0, 0};
+        auto fetch = [&](Pre& pr) {   // start the loads of the next tile of the walk
+            h_q[4] = hk * p.G + cur_gi;
+            r_q[4] = p.row_begin + cur_qt * BM;
+            prefetch(pr);
             advance();
-            stage_write(qd0, meta_s4[mb]);
-            __syncthreads();
-            // stores of the finished tile go out before this step's loads, so that
-            // waiting for those loads one step later never waits for younger stores
-            stage4(ds1, h_prev, r0_prev);
-            prefetch();
-            stage1(qd0, s, dp);
-            stage3(qd2, pb, dsb);
-            stage2(tail_c, s, dp, meta_s4[mb], ds0, pb, dsb);
-            h_prev = h_cur;
-            r0_prev = r0_cur;
-        }
+        };
+        auto shift = [&]() {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { h_q[k] = h_q[k + 1]; r_q[k] = r_q[k + 1]; }
+        };
+        f32x16 dp;
+        int b3 = 0;   // i % 3
 
-        // ---- drain: (3), (4) of the last tile
+        // Step i: stage tile i; P-waves do tile i; D-waves finish tile i-1 (dS, dK) and
+        // start tile i (dP); everyone copies dS^T(i-2) out.  Step n_iter only drains.
+        auto step = [&](int i, Pre& pr) {
+            const bool live = i < n_iter;
+            if (live) stage_write(pr, qd(b3), meta_s4[b3]);
+#ifndef LVX_EXP_NOBAR
+            __syncthreads();
+#endif
+            if (i >= 2) copy_out(dst(i & 1), h_q[0], r_q[0]);
+            if (i + 2 < n_iter) fetch(pr);
+            const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
+            if (!d_role) {
+                if (live) p_step(tail_c, qd(b3), meta_s4[b3], pbf(i & 1));
+            } else {
+                // VALU-heavy half first: it overlaps the S MFMAs of the P-wave on this SIMD,
+                // whose exp2 phase then overlaps the dK MFMAs issued here
+                if (i >= 1) d_step_ds(qd(b3p), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), dp);
+                if (live) d_step_dp(qd(b3), dp);
+            }
+            shift();
+            b3 = b3 == 2 ? 0 : b3 + 1;
+        };
+        // queue h_q/r_q: a tile enters at [4] when fetched; after k shifts it sits at
+        // [4-k].  Tile i is fetched two steps ahead, so at step i (before that
+        // step's shift) tile i is at [2], tile i-1 at [1], tile i-2 at [0].
+        fetch(preA);
+        shift();
+        if (n_iter > 1) fetch(preB);
+        shift();
+        for (int i = 0; i <= n_iter; i += 2) {
+            step(i, preA);
+            if (i + 1 <= n_iter) step(i + 1, preB);
+        }
         __syncthreads();
-        stage4(ds0, h_prev, r0_prev);
-        stage3(qd0, pb, dsb);
+        copy_out(dst((n_iter - 1) & 1), h_q[0], r_q[0]);
     };
     if (tail_block) run(std::true_type{});
     else run(std::false_type{});
 
-    // ---- epilogue: dK^T / dV^T rows = head-dim, cols = this wave's tokens
+    // ---- epilogue: rows of acc = head-dim, cols = this wave's tokens; P-waves hold dV^T, D-waves dK^T
     if (my_kv < p.Lkv) {
+        const Strides3 os = d_role ? p.dks : p.dvs;
+        void* optr = d_role ? p.dk : p.dv;
+        const int64_t off = b * os.b + hk * os.h + (int64_t)my_kv * os.s;
         if (p.dkv_accumulate) {
-            float* dkp = reinterpret_cast<float*>(p.dk) + b * p.dks.b + hk * p.dks.h + (int64_t)my_kv * p.dks.s;
-            float* dvp = reinterpret_cast<float*>(p.dv) + b * p.dvs.b + hk * p.dvs.h + (int64_t)my_kv * p.dvs.s;
+            float* op = reinterpret_cast<float*>(optr) + off;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
-                    f32x4 a = *reinterpret_cast<f32x4*>(dkp + d);
-                    f32x4 bb = *reinterpret_cast<f32x4*>(dvp + d);
+                    f32x4 a = *reinterpret_cast<f32x4*>(op + d);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        a[r] += dk[dt][4 * vg + r];
-                        bb[r] += dv[dt][4 * vg + r];
-                    }
-                    *reinterpret_cast<f32x4*>(dkp + d) = a;
-                    *reinterpret_cast<f32x4*>(dvp + d) = bb;
+                    for (int r = 0; r < 4; ++r) a[r] += acc[dt][4 * vg + r];
+                    *reinterpret_cast<f32x4*>(op + d) = a;
                 }
         } else {
-            uint16_t* dkp = reinterpret_cast<uint16_t*>(p.dk) + b * p.dks.b + hk * p.dks.h + (int64_t)my_kv * p.dks.s;
-            uint16_t* dvp = reinterpret_cast<uint16_t*>(p.dv) + b * p.dvs.b + hk * p.dvs.h + (int64_t)my_kv * p.dvs.s;
+            uint16_t* op = reinterpret_cast<uint16_t*>(optr) + off;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
-                    u32x2 a, bb;
-                    a[0] = pack_bf16(dk[dt][4 * vg], dk[dt][4 * vg + 1]);
-                    a[1] = pack_bf16(dk[dt][4 * vg + 2], dk[dt][4 * vg + 3]);
-                    bb[0] = pack_bf16(dv[dt][4 * vg], dv[dt][4 * vg + 1]);
-                    bb[1] = pack_bf16(dv[dt][4 * vg + 2], dv[dt][4 * vg + 3]);
-                    *reinterpret_cast<u32x2*>(dkp + d) = a;
-                    *reinterpret_cast<u32x2*>(dvp + d) = bb;
+                    u32x2 a;
+                    a[0] = pack_bf16(acc[dt][4 * vg], acc[dt][4 * vg + 1]);
+                    a[1] = pack_bf16(acc[dt][4 * vg + 2], acc[dt][4 * vg + 3]);
+                    *reinterpret_cast<u32x2*>(op + d) = a;
                 }
         }
     }
@@ -374,9 +393,9 @@ __global__ __launch_bounds__(256, 1) void bwd_kernel(const BwdParams p) {
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (masked)
-        hipLaunchKernelGGL(bwd_kernel<true>, dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(bwd_kernel<true>, dim3(grid), dim3(NT), 0, st, p);
     else
-        hipLaunchKernelGGL(bwd_kernel<false>, dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(bwd_kernel<false>, dim3(grid), dim3(NT), 0, st, p);
     return hipGetLastError();
 }
 

@@ -27,7 +27,7 @@ constexpr int TILE_ELEMS = (TM * LS > BK * LT) ? TM * LS : BK * LT;
 // ROW_CONTIG: memory is [k][row]; otherwise memory is [row][k].
 template <bool ROW_CONTIG>
 __device__ __forceinline__ void tile_load(u32x4 pre[4], const uint16_t* base, int64_t ld, int r0, int k0,
-                                          int R, int K, int tid) {
+                                          int R, int K, int tid, int tiled_m = 0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int c = tid + 256 * i;
@@ -36,7 +36,9 @@ __device__ __forceinline__ void tile_load(u32x4 pre[4], const uint16_t* base, in
             pre[i] = ldg16(base + (int64_t)r * ld + k, r < R && k < K);
         } else {
             const int k = k0 + (c >> 4), r = r0 + (c & 15) * 8;
-            pre[i] = ldg16(base + (int64_t)k * ld + r, k < K && r < R);
+            const int64_t off = tiled_m ? ((int64_t)(k >> 7) * tiled_m + (r >> 5)) * 4096 + (k & 127) * 32 + (r & 31)
+                                        : (int64_t)k * ld + r;
+            pre[i] = ldg16(base + off, k < K && r < R);
         }
     }
 }
@@ -104,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
         const int seg = s >= steps0 ? 1 : 0;
         const int k0 = (seg ? s - steps0 : s) * BK;
         const int kl = seg ? pr.K[1] : klen0;
-        tile_load<A_MCONTIG>(apre, pr.A[seg] + a_off, pr.lda[seg], m0, k0, p.M_ld, kl, tid);
+        tile_load<A_MCONTIG>(apre, pr.A[seg] + a_off, pr.lda[seg], m0, k0, p.M_ld, kl, tid, p.a_tiled_m);
         tile_load<B_NCONTIG>(bpre, pr.Bm[seg] + b_off, pr.ldb[seg], n0, k0, p.N, kl, tid);
     };
     if (steps > 0) prefetch(0);

@@ -61,8 +61,8 @@ struct BwdParams {
     const uint16_t* dout;
     const float* lse;
     const float* delta;
-    uint16_t* ds_ws;           // dS^T workspace [B*Hq][tokens padded to 128][ws_ld]
-    int64_t ws_ld;             // elements per token row (row window padded to 32)
+    uint16_t* ds_ws;           // dS^T workspace [B*Hq][token blocks][row tiles][128 tokens][32 rows]
+    int64_t ws_ld;             // elements per token block (row tiles * 4096)
     int64_t ws_bh;             // elements per (b, h) slab
     void* dk;
     void* dv;
@@ -109,6 +109,9 @@ struct GemmParams {
     int nbatch, batch_inner, b_group;
     int64_t a_batch, b_outer, b_inner, c_outer, c_inner;
     const int32_t* k_len;
+    // a_tiled_m > 0: A (stored [K][M]) is cut into contiguous [128 k][32 m] tiles,
+    // a_tiled_m of them per block of 128 k; lda is ignored
+    int a_tiled_m;
 };
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st);
