@@ -199,11 +199,40 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
     return static_cast<int>(launch_preprocess(p, static_cast<hipStream_t>(stream)));
 }
 
+// Work-groups of the backward are long (every step of a token block) and one
+// fits a CU, so a grid that is not a multiple of the CU count wastes up to one
+// whole round.  Splitting the steps of every token block over `S` work-groups
+// (which then add their dK/dV with atomics) evens that out; S is chosen to
+// minimise ceil(blocks * S / CUs) / S with ranges of at least 32 steps.
+static int choose_q_splits(int blocks, int steps) {
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n_cu = prop.multiProcessorCount;
+        if (n_cu <= 0) n_cu = 256;
+    }
+    int best = 1;
+    double best_cost = (double)((blocks + n_cu - 1) / n_cu);
+    for (int S = 2; S <= 8; ++S) {
+        if (steps / S < 32) break;
+        const double cost = (double)(((int64_t)blocks * S + n_cu - 1) / n_cu) / S;
+        if (cost < best_cost * 0.97) { best_cost = cost; best = S; }
+    }
+    return best;
+}
+
+static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
+    return (size_t)2 * s->B * s->Lkv * s->Hkv * s->D * sizeof(float);
+}
+
 size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
     if (!s || row_count <= 0) return 0;
     const size_t tokens = ((size_t)s->Lkv + 127) / 128 * 128;
     const size_t rows = ((size_t)row_count + 31) / 32 * 32;
-    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t);
+    // dS^T tiles, then fp32 dK/dV scratch for the split-steps mode with bf16 outputs
+    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s);
 }
 
 int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
@@ -241,16 +270,50 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.B = s->B; p.Hq = s->Hq; p.Hkv = s->Hkv; p.Lq = s->Lq; p.Lkv = s->Lkv; p.G = s->Hq / s->Hkv;
     p.row_begin = row_begin; p.row_end = row_begin + row_count;
     p.n_kv_blocks = (s->Lkv + 127) / 128;
-    p.total_wg = s->B * s->Hkv * p.n_kv_blocks;
-    p.dkv_accumulate = dkv_accumulate;
     p.scale = s->scale; p.scale_log2e = s->scale * LOG2E;
     const int64_t tokens = (int64_t)p.n_kv_blocks * 128;
     const int64_t rows = ((int64_t)row_count + 31) / 32 * 32;
     p.ds_ws = static_cast<uint16_t*>(workspace);
     p.ws_ld = rows * 128;          // one token block: (rows / 32) tiles of 128 x 32
     p.ws_bh = tokens * rows;
+
+    const int blocks = s->B * s->Hkv * p.n_kv_blocks;
+    const int steps = p.G * (int)(rows / 32);
+    p.q_splits = choose_q_splits(blocks, steps);
+    p.split_steps = (steps + p.q_splits - 1) / p.q_splits;
+    p.total_wg = blocks * p.q_splits;
+    p.dkv_mode = dkv_accumulate ? 1 : 0;
+    float* scratch = nullptr;
+    const int64_t dkv_elems = (int64_t)s->B * s->Lkv * s->Hkv * s->D;
+    if (p.q_splits > 1) {
+        p.dkv_mode = 2;
+        if (!dkv_accumulate) {
+            // bf16 outputs: sum the splits in an fp32 scratch [2][B, Lkv, Hkv, D], round once afterwards
+            scratch = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                               (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t));
+            FillParams f{reinterpret_cast<uint32_t*>(scratch), (int64_t)(dkv_scratch_bytes(s) / 16)};
+            hipError_t ez = launch_zero(f, st);
+            if (ez != hipSuccess) return static_cast<int>(ez);
+            p.dk = scratch;
+            p.dv = scratch + dkv_elems;
+            p.dks = p.dvs = Strides3{(int64_t)s->Lkv * s->Hkv * s->D, (int64_t)s->D, (int64_t)s->Hkv * s->D};
+        }
+    }
     hipError_t e = launch_bwd(p, s->kv_start != nullptr, st);
     if (e != hipSuccess) return static_cast<int>(e);
+    if (scratch) {
+        for (int i = 0; i < 2; ++i) {
+            const lvx_tensor* t = i ? dv : dk;
+            // scratch memory order is [B, Lkv, Hkv, D]: cast with (H, L) = (Lkv, Hkv)
+            CastParams cp{};
+            cp.src = scratch + i * dkv_elems;
+            cp.dst = static_cast<uint16_t*>(t->ptr);
+            cp.ds = Strides3{t->stride_b, t->stride_s, t->stride_h};
+            cp.B = s->B; cp.H = s->Lkv; cp.L = s->Hkv;
+            e = launch_cast(cp, st);
+            if (e != hipSuccess) return static_cast<int>(e);
+        }
+    }
 
     // dQ[b, h, rows, :] = dS^T[b, h]^T (rows x tokens) * K[b, h / G] (tokens x D), scale already in dS
     GemmParams g{};

@@ -71,8 +71,9 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
-    const int kblk = wid % p.n_kv_blocks;
-    const int bh = wid / p.n_kv_blocks;
+    const int sp = wid % p.q_splits;
+    const int kblk = (wid / p.q_splits) % p.n_kv_blocks;
+    const int bh = wid / (p.q_splits * p.n_kv_blocks);
     const int hk = bh % p.Hkv;
     const int b = bh / p.Hkv;
 
@@ -104,8 +105,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
 
+    // steps of this work-group: a contiguous range of the (head, row tile) list
     const int n_qtiles = (p.row_end - p.row_begin + BM - 1) / BM;
-    const int n_iter = (kvb < kv_len) ? p.G * n_qtiles : 0;
+    const int it_lo = sp * p.split_steps;
+    const int n_iter = (kvb < kv_len) ? max(0, min(p.split_steps, p.G * n_qtiles - it_lo)) : 0;
     const float c = p.scale_log2e;
 
     // staging role of this thread: threads 0..255 carry Q, 256..511 carry dO; two
@@ -137,14 +140,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // workspace tile (b, h, token block, row tile): [128 tokens][32 rows], 8 KB, contiguous
     uint16_t* ws_lane = p.ds_ws + (int64_t)kblk * p.ws_ld + cp_token * BM + cp_part * 8;
 
-    // token blocks of one kv head walk the (head, row tile) list from different
-    // starting points, which spreads their reads of Q / dO over the L2
-    int cur_gi = 0, cur_qt = 0;
-    if (n_iter > 0) {
-        const int it_shift = (int)(((int64_t)kblk * 7) % n_iter);
-        cur_gi = it_shift / n_qtiles;
-        cur_qt = it_shift % n_qtiles;
-    }
+    int cur_gi = it_lo / n_qtiles, cur_qt = it_lo % n_qtiles;
 
     // Every load is unconditional: rows past the window are clamped to its last
     // row (their LSE is forced to +inf, so P = 0 and nothing they carry reaches a
@@ -356,11 +352,35 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     else run(std::false_type{});
 
     // ---- epilogue: rows of acc = head-dim, cols = this wave's tokens; P-waves hold dV^T, D-waves dK^T
-    if (my_kv < p.Lkv) {
+    if (p.dkv_mode == 2) {
+        // Several work-groups (ranges of steps) share this token block: add with
+        // atomics.  The accumulator has tokens along the lanes; it is turned
+        // through LDS so that each atomic instruction covers 64 consecutive
+        // floats (two full lines) of one token row.
+        __syncthreads();   // the staging buffers are free now
+        if (n_iter > 0) {
+            constexpr int EPS = D + 1;
+            float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EPS);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) ep[l32 * EPS + dt * 32 + acc_row(v, g)] = acc[dt][v];
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): this wave's LDS writes have landed
+            const Strides3 os = d_role ? p.dks : p.dvs;
+            float* obase = reinterpret_cast<float*>(d_role ? p.dk : p.dv) + b * os.b + hk * os.h;
+            for (int t = 0; t < 32; ++t) {
+                const int token = kvb + 32 * slice + t;
+                if (token >= p.Lkv) break;
+                float* op = obase + (int64_t)token * os.s;
+                unsafeAtomicAdd(op + lane, ep[t * EPS + lane]);
+                unsafeAtomicAdd(op + 64 + lane, ep[t * EPS + 64 + lane]);
+            }
+        }
+    } else if (my_kv < p.Lkv) {
         const Strides3 os = d_role ? p.dks : p.dvs;
         void* optr = d_role ? p.dk : p.dv;
         const int64_t off = b * os.b + hk * os.h + (int64_t)my_kv * os.s;
-        if (p.dkv_accumulate) {
+        if (p.dkv_mode == 1) {
             float* op = reinterpret_cast<float*>(optr) + off;
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)

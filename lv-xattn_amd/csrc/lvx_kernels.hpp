@@ -73,8 +73,15 @@ struct BwdParams {
     int B, Hq, Hkv, Lq, Lkv, G;
     int row_begin, row_end;
     int n_kv_blocks, total_wg;
-    int dkv_accumulate;
+    int q_splits;              // work-groups sharing one token block, each taking a range of steps
+    int split_steps;           // steps (32-row tiles x heads of the group) per split
+    int dkv_mode;              // 0: store bf16, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1)
     float scale, scale_log2e;
+};
+
+struct FillParams {
+    uint32_t* dst;             // 16-byte aligned
+    int64_t n16;               // number of 16-byte chunks to zero
 };
 
 struct CastParams {
@@ -119,6 +126,7 @@ hipError_t launch_merge(const MergeParams& p, hipStream_t st);
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st);
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);
 hipError_t launch_cast(const CastParams& p, hipStream_t st);
+hipError_t launch_zero(const FillParams& p, hipStream_t st);
 // a_mcontig: A is stored [K][M] (m contiguous); b_ncontig: B is stored [K][N].
 hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st);
 

@@ -128,6 +128,13 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
+// zero fill (a kernel rather than hipMemsetAsync, so that callers may capture the stream)
+__global__ __launch_bounds__(256) void zero_kernel(const FillParams p) {
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < p.n16; i += (int64_t)gridDim.x * 256)
+        reinterpret_cast<u32x4*>(p.dst)[i] = z;
+}
+
 inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 
 }  // namespace
@@ -143,6 +150,13 @@ hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
     hipLaunchKernelGGL(preprocess_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_zero(const FillParams& p, hipStream_t st) {
+    if (p.n16 <= 0) return hipSuccess;
+    const int grid = (int)((p.n16 + 255) / 256 < 4096 ? (p.n16 + 255) / 256 : 4096);
+    hipLaunchKernelGGL(zero_kernel, dim3(grid), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
