@@ -58,7 +58,10 @@ constexpr int PB_ELEMS = 4 * 2 * 64 * 8;       // P hand-over: [slice][half][lan
 constexpr int OFF_QD = 0;                      // x3
 constexpr int OFF_DST = OFF_QD + 3 * QD_ELEMS; // x2
 constexpr int OFF_PB = OFF_DST + 2 * DST_ELEMS;  // x2
-constexpr int SMEM_ELEMS = OFF_PB + 2 * PB_ELEMS;
+constexpr int LOOP_ELEMS = OFF_PB + 2 * PB_ELEMS;
+constexpr int EPS = D + 1;                          // row stride (floats) of the epilogue's transposed tile
+constexpr int EPI_ELEMS = 8 * 32 * EPS * 2;         // 8 waves x [32 tokens][128 + 1] floats, in uint16 units
+constexpr int SMEM_ELEMS = LOOP_ELEMS > EPI_ELEMS ? LOOP_ELEMS : EPI_ELEMS;
 
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -154,12 +157,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         bool ok;
     };
     Pre preA{}, preB{};
-    int exp_loads = 0;
     auto prefetch = [&](Pre& pr) {
-#ifdef LVX_EXP_NOLOAD
-        if (exp_loads >= 2) return;
-        ++exp_loads;
-#endif
         const int h = hk * p.G + cur_gi;
         const int r0 = p.row_begin + cur_qt * BM;
         const uint16_t* base = g_base + h * g_hs + s_chunk * 8;
@@ -179,9 +177,6 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
     };
     auto stage_write = [&](const Pre& pr, uint16_t* qd, u32x4* meta) {
-#ifdef LVX_EXP_NOSTAGE
-        if (pr.m == 0x12345678u)
-#endif
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             *reinterpret_cast<u32x4*>(qd + stage_off + 16 * i * QS) = pr.d[i];
@@ -197,9 +192,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // the finished dS^T tile goes to HBM as one contiguous 8 KB block
     auto copy_out = [&](const uint16_t* dst, int h, int r0) {
         uint16_t* gp = ws_lane + ((int64_t)b * p.Hq + h) * p.ws_bh + (int64_t)((r0 - p.row_begin) / BM) * (BN * BM);
-#ifndef LVX_EXP_NOSTORE
         *reinterpret_cast<u32x4*>(gp) = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
-#endif
     };
 
     // ---- P-wave: S = Q K_w^T, P = exp2(S*c - LSE*log2e) (masked), hand P over, dV_w^T += dO^T P
@@ -317,9 +310,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         auto step = [&](int i, Pre& pr) {
             const bool live = i < n_iter;
             if (live) stage_write(pr, qd(b3), meta_s4[b3]);
-#ifndef LVX_EXP_NOBAR
             __syncthreads();
-#endif
             if (i >= 2) copy_out(dst(i & 1), h_q[0], r_q[0]);
             if (i + 2 < n_iter) fetch(pr);
             const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
@@ -359,7 +350,6 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // floats (two full lines) of one token row.
         __syncthreads();   // the staging buffers are free now
         if (n_iter > 0) {
-            constexpr int EPS = D + 1;
             float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EPS);
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)

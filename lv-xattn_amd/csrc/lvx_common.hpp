@@ -25,12 +25,7 @@ constexpr int WAVE = 64;
 // Slot (g, e) of A multiplies slot (g, e) of B; which logical k a slot stands
 // for is the caller's choice as long as both operands agree.
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-#ifdef LVX_EXP_NOMFMA
-    c[0] += __builtin_bit_cast(u32x4, a)[0] * 1e-30f + __builtin_bit_cast(u32x4, b)[1] * 1e-30f;
-    return c;
-#else
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-#endif
 }
 
 // Row of accumulator register v for lane-half g (see above).
@@ -102,10 +97,6 @@ __device__ __forceinline__ int tr_lane_offset(int lane, int stride, bool permute
 }
 
 __device__ __forceinline__ bf16x8 lds_operand_tr(const uint16_t* p, int half_offset) {
-#ifdef LVX_EXP_NOTR
-    const u32x4 z = {(uint32_t)(uintptr_t)p, 0x3f803f80u, 0x3f803f80u, (uint32_t)half_offset};
-    return __builtin_bit_cast(bf16x8, z);
-#endif
     const u32x2 a = lds_read_tr16(p), b = lds_read_tr16(p + half_offset);
     const u32x4 u = {a[0], a[1], b[0], b[1]};
     return as_bf16x8(u);
