@@ -21,8 +21,11 @@
 // K and V are both staged row-major: K [64][128+8] (68-dword rows: the 16-byte
 // operand reads of 16 consecutive lanes hit 64 distinct banks), V [64][128+16]
 // (72-dword rows: the 8 rows x 16 dwords a transposing read touches tile the
-// banks twice).  The next tile's global loads are in flight while the current
-// one is consumed.
+// banks twice).  The LDS tiles are double-buffered: while tile t is consumed,
+// tile t+1 moves from registers into the other buffer and tile t+2's global
+// loads are issued, with one barrier per tile.  Loads past the end of the key
+// range are clamped to its last row (those keys are masked out of S), so the
+// loop body has no divergent branch.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -38,8 +41,8 @@ constexpr int BIG = 0x3fffffff;
 
 template <bool MASKED>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * VS];
+    __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * KS];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * VS];
     __shared__ int red[4][4];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
@@ -108,18 +111,20 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     const int off_vT = tr_lane_offset(lane, VS, true);   // V^T operand, keys in accumulator order
 
     u32x4 kpre[4], vpre[4];
+    const int ld_row = tid >> 4, ld_col = (tid & 15) * 8;   // this thread's chunk of rows ld_row + 16 i
     auto prefetch = [&](int kv0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i;
-            const int kv = kv0 + (c >> 4);
-            kpre[i] = ldg16(kbase + (int64_t)kv * p.ks.s + (c & 15) * 8, kv < kv_hi);
+            const int kv = min(kv0 + ld_row + 16 * i, kv_hi - 1);
+            kpre[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kv * p.ks.s + ld_col);
+            vpre[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kv * p.vs.s + ld_col);
         }
+    };
+    auto stage = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i;
-            const int kv = kv0 + (c >> 4);
-            vpre[i] = ldg16(vbase + (int64_t)kv * p.vs.s + (c & 15) * 8, kv < kv_hi);
+            *reinterpret_cast<u32x4*>(&Ks2[buf][(ld_row + 16 * i) * KS + ld_col]) = kpre[i];
+            *reinterpret_cast<u32x4*>(&Vs2[buf][(ld_row + 16 * i) * VS + ld_col]) = vpre[i];
         }
     };
 
@@ -133,19 +138,18 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
     const int t_begin = (hi > lo) ? lo / BN : 0;
     const int t_end = (hi > lo) ? (hi + BN - 1) / BN : 0;
-    if (t_end > t_begin) prefetch(t_begin * BN);
+    if (t_end > t_begin) {
+        prefetch(t_begin * BN);
+        stage(0);
+        __syncthreads();
+        prefetch(min(t_begin + 1, t_end - 1) * BN);
+    }
 
     for (int t = t_begin; t < t_end; ++t) {
         const int kv0 = t * BN;
-        __syncthreads();   // everyone is done reading the previous tile
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int cidx = tid + 256 * i;
-            *reinterpret_cast<u32x4*>(&Ks[(cidx >> 4) * KS + (cidx & 15) * 8]) = kpre[i];
-            *reinterpret_cast<u32x4*>(&Vs[(cidx >> 4) * VS + (cidx & 15) * 8]) = vpre[i];
-        }
-        __syncthreads();
-        if (t + 1 < t_end) prefetch(kv0 + BN);
+        const int buf = (t - t_begin) & 1;
+        const uint16_t* Ks = Ks2[buf];
+        const uint16_t* Vs = Vs2[buf];
 
         // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows
         f32x16 s0, s1;
@@ -171,7 +175,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         float mx = fmaxf(s0[0], s1[0]);
 #pragma unroll
         for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(s0[v], s1[v]));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        {   // other half of the wave holds the other 32 keys of the same text row
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+        }
         const float m_new = fmaxf(m_i, mx);
         const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
         const float alpha = __builtin_amdgcn_exp2f(m_i * c - mc);
@@ -200,10 +207,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
             pb[2 + j] = as_bf16x8(u1);
         }
 
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {   // the running max moved for some row
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[dt][v] *= alpha;
+                for (int v = 0; v < 16; ++v) acc[dt][v] *= alpha;
+        }
 
         // O^T += V^T P^T
 #pragma unroll
@@ -213,6 +222,14 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
                 const bf16x8 a = lds_operand_tr(&Vs[off_vT + 16 * j * VS + dt * 32], 8 * VS);
                 acc[dt] = mfma32(a, pb[j], acc[dt]);
             }
+
+        // tile t+1 (in registers since the previous iteration) goes to the other
+        // buffer, whose last readers finished before the previous barrier
+        if (t + 1 < t_end) {
+            stage(buf ^ 1);
+            __syncthreads();
+            prefetch(min(t + 2, t_end - 1) * BN);
+        }
     }
 
     // epilogue: the two lane halves hold partial row sums of the same row
