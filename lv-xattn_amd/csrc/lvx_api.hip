@@ -365,8 +365,8 @@ static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch = 1) {
     g.nbatch = nbatch;
     if (g.batch_inner < 1) g.batch_inner = 1;
     if (g.b_group < 1) g.b_group = 1;
-    g.tiles_m = (M + 127) / 128;
-    g.tiles_n = (N + 127) / 128;
+    g.tiles_m = (M + 64 * GEMM_WM - 1) / (64 * GEMM_WM);
+    g.tiles_n = (N + 64 * GEMM_WN - 1) / (64 * GEMM_WN);
     g.total_wg = nprob * nbatch * g.tiles_m * g.tiles_n;
 }
 

@@ -91,6 +91,15 @@ struct CastParams {
     int B, H, L;
 };
 
+// MFMA tiles (32 x 32) per wave along M and N; a work-group is 2 x 2 waves,
+// so its tile of C is (64 GEMM_WM) x (64 GEMM_WN).
+#ifndef GEMM_WM
+#define GEMM_WM 4
+#endif
+#ifndef GEMM_WN
+#define GEMM_WN 2
+#endif
+
 // One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].
 struct GemmProblem {
     const uint16_t* A[2];
