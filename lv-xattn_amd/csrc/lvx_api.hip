@@ -353,7 +353,7 @@ int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_
 static int check_gemm_ptr(const void* p, int64_t ld) {
     if (!p) return LVX_ERR_NULL;
     if (!aligned16(p) || (ld % 8) != 0) return LVX_ERR_ALIGN;
-    if (ld <= 0) return LVX_ERR_SHAPE;
+    if (ld <= 0 || ld >= (1 << 21)) return LVX_ERR_SHAPE;   // 32-bit byte offsets inside a tile
     return LVX_OK;
 }
 
@@ -365,9 +365,6 @@ static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch = 1) {
     g.nbatch = nbatch;
     if (g.batch_inner < 1) g.batch_inner = 1;
     if (g.b_group < 1) g.b_group = 1;
-    g.tiles_m = (M + 64 * GEMM_WM - 1) / (64 * GEMM_WM);
-    g.tiles_n = (N + 64 * GEMM_WN - 1) / (64 * GEMM_WN);
-    g.total_wg = nprob * nbatch * g.tiles_m * g.tiles_n;
 }
 
 extern "C" {

@@ -1,18 +1,27 @@
 // bf16 GEMM for the K/V recompute (K = X W_k, V = X W_v), its input gradient
 // (dX = dK W_k^T + dV W_v^T, one GEMM whose contraction runs over two operand
-// pairs) and the weight gradients (dW = X^T dK).  fp32 accumulate on
-// v_mfma_f32_32x32x16_bf16, bf16 output.
+// pairs), the weight gradients (dW = X^T dK) and the batched dQ = dS K of the
+// attention backward.  fp32 accumulate on v_mfma_f32_32x32x16_bf16, bf16 output.
 //
-// A work-group computes a (64 WM) x (64 WN) tile of C with 4 waves in a 2 x 2
-// grid, each wave WM x WN MFMA tiles, stepping 64 along the contraction.  The
-// default is 256 x 128 (wave tile 128 x 64): every LDS operand read then feeds
-// 2 or 4 MFMAs, which keeps the LDS pipe well below the MFMA pipe.  An operand
-// whose memory has the contraction index contiguous is staged as [rows][64+8]
-// and read with 16-byte LDS reads; an operand whose memory has the OTHER index
-// contiguous is staged exactly as it lies in memory, [64 k][rows+32], and read
-// with the transposing LDS read - nothing is transposed on the way in.  The
-// MFMA computes C^T (A operand = rows of the B tile), so a lane ends up with 4
-// consecutive columns of one C row and stores 8 bytes.
+// Structure (8 waves, two per SIMD, in lock-step "ping-pong"):
+//  * Operand tiles go from global memory straight into LDS with
+//    global_load_lds_dwordx4 (no staging registers), NS stages of 32 k deep, so
+//    a tile is requested NS-1 stages before it is used.
+//  * Waves 0-3 and waves 4-7 (one of each per SIMD) run the same loop half a
+//    stage apart: while one set issues the 16 MFMAs of a stage from registers,
+//    the other set fetches its operands of the next stage from LDS and issues
+//    its share of the global loads; a work-group barrier after every phase
+//    keeps the two sets alternating, so the MFMA pipe of every SIMD always has
+//    one wave feeding it and the LDS / memory latency of the other is hidden.
+//  * The direct-to-LDS load writes 64 lanes x 16 bytes contiguously, so tiles
+//    cannot be padded; bank conflicts are avoided by permuting 16-byte chunks
+//    (an XOR of the chunk index with row bits), applied on the global-address
+//    side when loading and on the LDS-address side when reading.
+//  * An operand whose memory has the contraction index contiguous is read
+//    with 16-byte LDS reads; one whose memory has the OTHER index contiguous
+//    is kept as it lies, [k][rows], and read with the transposing LDS read.
+//  * The MFMA computes C^T (A operand = rows of the B tile), so a lane ends up
+//    with 4 consecutive columns of one C row and stores 8 bytes.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -20,95 +29,99 @@ namespace lvx {
 
 namespace {
 
-constexpr int BK = 64;
-constexpr int LS = BK + 8;     // row stride of a [row][k] tile (36 dwords)
-// a tile of ROWS rows: [ROWS][LS] or [BK][ROWS + 32] (row stride = 16 mod 64 dwords)
-constexpr int tile_elems(int rows) { return rows * LS > BK * (rows + 32) ? rows * LS : BK * (rows + 32); }
+constexpr int BK = 32;                 // contraction depth of one stage
+__device__ uint32_t zero_chunk[4];     // source of the chunks past the end of a contraction
 
-// Global -> LDS staging of one operand tile (ROWS rows x 64 k), ROWS/32 chunks of
-// 16 bytes per thread.  ROW_CONTIG: memory is [k][row]; otherwise [row][k].
-// Every load is `uniform stage base + per-thread 32-bit byte offset`: the
-// offsets are computed once (rows past the end are clamped onto a valid row;
-// their products are never stored), the base advances by one k-step per
-// stage, so the steady-state loop issues bare loads with no address arithmetic.
-// Only the last stage of a contraction segment, when it is partial, re-derives
-// clamped offsets and zeroes the chunks whose k lies past the end.
+// 64 lanes x 16 bytes from global memory to the 1 KiB of LDS at byte address
+// lds_byte (wave-uniform); lane i lands at lds_byte + 16 i.  Counted by vmcnt.
+__device__ __forceinline__ void dma16(const char* sbase, uint32_t voff, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_addr(const char* addr, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte), "v"(addr) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void phase_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One operand's part of a stage: ROWS rows x 32 k, unpadded, in wave-chunks of
+// 1 KiB (what one global_load_lds_dwordx4 writes).
+//   !ROW_CONTIG (memory [row][k]): LDS row r at r*64 B; its 16-byte chunk c
+//       (k = 8c..8c+7) sits at position c ^ ((r >> 2) & 3).
+//    ROW_CONTIG (memory [k][row]): LDS k-row at k*ROWS*2 B; its chunk q (rows
+//       8q..8q+7) sits at position q ^ ((k & 3) << 2).
 template <bool ROW_CONTIG, int ROWS>
-struct TileLoader {
-    static constexpr int NCH = ROWS / 32;
-    static constexpr int CPR = ROWS / 8;      // chunks per k row of a [k][row] tile
-    static constexpr int LT = ROWS + 32;
-    uint32_t voff[NCH];
-    u32x4 pre[NCH];
-    uint32_t kstep_bytes;                      // byte distance of one k row (ROW_CONTIG) or 2
+struct Region {
+    static constexpr int BYTES = ROWS * BK * 2;
+    static constexpr int CHUNKS = BYTES / 1024;
+    static constexpr int LPR = ROWS / 8;          // lanes per k-row (ROW_CONTIG)
 
-    __device__ __forceinline__ static int kpos(int c) { return ROW_CONTIG ? c / CPR : (c & 7) * 8; }
-
-    __device__ __forceinline__ void setup(int64_t ld, int r0, int R, int tid, int tiled_m) {
-        kstep_bytes = ROW_CONTIG ? (tiled_m ? 64u : (uint32_t)ld * 2u) : 2u;
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = tid + 256 * i;
-            if (!ROW_CONTIG) {
-                const int r = min(r0 + (c >> 3), R - 1) - r0;
-                voff[i] = (uint32_t)r * (uint32_t)ld * 2u + (uint32_t)(c & 7) * 16u;
-            } else if (tiled_m) {
-                const int r = min(r0 + (c % CPR) * 8, R - 8);
-                voff[i] = (uint32_t)((c / CPR) * 32 + (r >> 5) * 4096 + (r & 31)) * 2u;
-            } else {
-                const int r = min(r0 + (c % CPR) * 8, R - 8) - r0;
-                voff[i] = (uint32_t)(c / CPR) * (uint32_t)ld * 2u + (uint32_t)r * 2u;
-            }
+    // what lane `lane` of the wave loading chunk `ch` fetches: byte offset from the
+    // stage base of the operand, and the k position inside the stage
+    __device__ __forceinline__ static uint32_t src(int ch, int lane, int r0, int R, int64_t ld, int tiled_m,
+                                                   int& kpos) {
+        if (!ROW_CONTIG) {
+            const int row = 16 * ch + (lane >> 2);
+            const int c = (lane & 3) ^ ((lane >> 4) & 3);
+            kpos = c * 8;
+            return (uint32_t)(min(r0 + row, R - 1) - r0) * (uint32_t)ld * 2u + (uint32_t)c * 16u;
         }
+        const int k = ch * (64 / LPR) + lane / LPR;
+        const int q = (lane % LPR) ^ ((k & 3) << 2);
+        kpos = k;
+        const int r = min(r0 + q * 8, R - 8);
+        if (tiled_m) return (uint32_t)(k * 32 + (r >> 5) * 4096 + (r & 31)) * 2u;
+        return (uint32_t)k * (uint32_t)ld * 2u + (uint32_t)(r - r0) * 2u;
     }
 
-    // base: address of (row r0, k0) of the operand (tiled: of the k0 tile row); krem = K - k0 > 0
-    __device__ __forceinline__ void load(const char* base, int krem, int tid) {
-        if (krem >= BK) {
-#pragma unroll
-            for (int i = 0; i < NCH; ++i) pre[i] = *reinterpret_cast<const u32x4*>(base + voff[i]);
+    // per-lane LDS byte offsets for the operand reads of a wave whose first
+    // 32-row tile in the region is tile j0 (W tiles per wave).
+    //  !ROW_CONTIG: rd[kk] for k-step kk; add tile * 2048
+    //   ROW_CONTIG: rd[t] for tile t; add kk * 16 * ROWS * 2 (+ 4 * ROWS * 2 for the second half)
+    template <int W>
+    __device__ __forceinline__ static void read_offsets(uint32_t* rd, int j0, int lane) {
+        if (!ROW_CONTIG) {
+            const int l32 = lane & 31, g = lane >> 5, s = (l32 >> 2) & 3;
+            rd[0] = (uint32_t)(j0 * 2048 + l32 * 64 + ((g ^ s) * 16));
+            rd[1] = (uint32_t)(j0 * 2048 + l32 * 64 + (((2 + g) ^ s) * 16));
         } else {
+            const int r = (lane & 15) >> 2, t = lane & 3, u = (lane >> 4) & 1, g = lane >> 5;
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) {
-                const int kp = kpos(tid + 256 * i);
-                const uint32_t back = (uint32_t)kp * kstep_bytes;
-                pre[i] = *reinterpret_cast<const u32x4*>(base + (kp < krem ? voff[i] : voff[i] - back));
-            }
+            for (int i = 0; i < W; ++i)
+                rd[i] = (uint32_t)((8 * g + r) * ROWS * 2 + 64 * ((j0 + i) ^ r) + (2 * u + (t >> 1)) * 16 + (t & 1) * 8);
         }
     }
+    static constexpr int NRD(int W) { return ROW_CONTIG ? W : 2; }
 
-    __device__ __forceinline__ void store(uint16_t* lds, int krem, int tid) {
-        if (krem < BK) {
-            const u32x4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int i = 0; i < NCH; ++i)
-                if (kpos(tid + 256 * i) >= krem) pre[i] = z;
-        }
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = tid + 256 * i;
-            if (!ROW_CONTIG)
-                *reinterpret_cast<u32x4*>(&lds[(c >> 3) * LS + (c & 7) * 8]) = pre[i];
-            else
-                *reinterpret_cast<u32x4*>(&lds[(c / CPR) * LT + (c % CPR) * 8]) = pre[i];
-        }
+    // operand (tile t of the wave, k-step kk) from the stage at LDS byte offset `base`
+    __device__ __forceinline__ static bf16x8 operand(const char* lds, uint32_t base, const uint32_t* rd, int t, int kk) {
+        if (!ROW_CONTIG) return *reinterpret_cast<const bf16x8*>(lds + base + rd[kk] + t * 2048);
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(lds + base + rd[t] + kk * 16 * ROWS * 2);
+        return lds_operand_tr(p, 4 * ROWS);
     }
 };
 
-// MFMA operand for tile rows row0..row0+31 and k-step kk (16 values of k).
-template <bool ROW_CONTIG, int ROWS>
-__device__ __forceinline__ bf16x8 tile_operand(const uint16_t* lds, int row0, int kk, int lane, int tr_off) {
-    constexpr int LT = ROWS + 32;
-    if (!ROW_CONTIG)
-        return *reinterpret_cast<const bf16x8*>(&lds[(row0 + (lane & 31)) * LS + kk * 16 + (lane >> 5) * 8]);
-    return lds_operand_tr(&lds[tr_off + row0 + kk * 16 * LT], 4 * LT);
-}
-
-template <bool A_MCONTIG, bool B_NCONTIG, int WM, int WN>
-__global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
-    constexpr int TM = 64 * WM, TN = 64 * WN;
-    __shared__ __attribute__((aligned(16))) uint16_t As[tile_elems(TM)];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[tile_elems(TN)];
+// GM x GN waves, each WM x WN MFMA tiles: work-group tile (32 WM GM) x (32 WN GN).
+template <bool A_MCONTIG, bool B_NCONTIG, int GM, int GN, int WM, int WN, int NS>
+__global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
+    static_assert(GM * GN == 8, "8 waves");
+    constexpr int TM = 32 * WM * GM, TN = 32 * WN * GN;
+    using RA = Region<A_MCONTIG, TM>;
+    using RB = Region<B_NCONTIG, TN>;
+    constexpr int STAGE = RA::BYTES + RB::BYTES;
+    constexpr int LPG = (RA::CHUNKS + RB::CHUNKS) / 8;     // loads per wave per stage
+    constexpr int LPG_A = RA::CHUNKS / 8;
+    static_assert(RA::CHUNKS % 8 == 0 && RB::CHUNKS % 8 == 0, "chunks split evenly over 8 waves");
+    constexpr int NRA = RA::NRD(WM), NRB = RB::NRD(WN);
+    __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
@@ -125,12 +138,65 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
     uint16_t* const Cz = pr.C + zo * p.c_outer + zi * p.c_inner;
     int klen0 = pr.K[0];
     if (p.k_len) klen0 = min(klen0, p.k_len[zo]);
+    const int klen1 = pr.nseg > 1 ? pr.K[1] : 0;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
-    const int wm = wave & 1, wn = wave >> 1;
-    const int tr_off_a = tr_lane_offset(lane, TM + 32, false);
-    const int tr_off_b = tr_lane_offset(lane, TN + 32, false);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int set = wave >> 2;
+    const int wm = wave % GM, wn = wave / GM;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+
+    // ---- global -> LDS: this wave's LPG chunks of every stage
+    const int64_t lda = pr.lda[0], ldb = pr.ldb[0];
+    uint32_t voff[LPG];
+    int kpos[LPG];
+#pragma unroll
+    for (int j = 0; j < LPG; ++j) {
+        const int ch = wave + 8 * j;
+        if (j < LPG_A) voff[j] = RA::src(ch, lane, m0, p.M_ld, lda, p.a_tiled_m, kpos[j]);
+        else voff[j] = RB::src(ch - RA::CHUNKS, lane, n0, p.N, ldb, 0, kpos[j]);
+    }
+    const char* abase[2];
+    const char* bbase[2];
+#pragma unroll
+    for (int sg = 0; sg < 2; ++sg) {
+        const int ss = sg < pr.nseg ? sg : 0;
+        abase[sg] = reinterpret_cast<const char*>(pr.A[ss] + a_off);
+        if (!p.a_tiled_m) abase[sg] += (A_MCONTIG ? (int64_t)m0 : (int64_t)m0 * lda) * 2;
+        bbase[sg] = reinterpret_cast<const char*>(pr.Bm[ss] + b_off) + (B_NCONTIG ? (int64_t)n0 : (int64_t)n0 * ldb) * 2;
+    }
+    const int64_t a_kstride = A_MCONTIG ? lda * BK * 2 : BK * 2;   // bytes per stage (untiled)
+    const int64_t b_kstride = B_NCONTIG ? ldb * BK * 2 : BK * 2;
+    const int steps0 = (klen0 + BK - 1) / BK;
+    const int steps = steps0 + (klen1 + BK - 1) / BK;
+
+    auto issue = [&](int s) {     // loads of stage s into ring slot s % NS
+        const int sg = s >= steps0 ? 1 : 0;
+        const int ks = sg ? s - steps0 : s;
+        const int krem = (sg ? klen1 : klen0) - ks * BK;
+        const char* ab = abase[sg] + ks * a_kstride;
+        if (A_MCONTIG && p.a_tiled_m)   // tiled A: [k / 128][m / 32][128 k][32 m]
+            ab = abase[sg] + ((int64_t)(ks >> 2) * p.a_tiled_m * 4096 + (ks & 3) * (BK * 32)) * 2;
+        const char* bb = bbase[sg] + ks * b_kstride;
+        const uint32_t slot = lds0 + (uint32_t)(s % NS) * STAGE + (uint32_t)wave * 1024u;
+        if (krem >= BK) {
+#pragma unroll
+            for (int j = 0; j < LPG; ++j)
+                dma16(j < LPG_A ? ab : bb, voff[j], slot + (j < LPG_A ? j * 8192 : RA::BYTES + (j - LPG_A) * 8192));
+        } else {
+            const char* zc = reinterpret_cast<const char*>(zero_chunk);
+#pragma unroll
+            for (int j = 0; j < LPG; ++j) {
+                const char* src = (j < LPG_A ? ab : bb) + voff[j];
+                dma16_addr(kpos[j] < krem ? src : zc, slot + (j < LPG_A ? j * 8192 : RA::BYTES + (j - LPG_A) * 8192));
+            }
+        }
+    };
+
+    // ---- LDS -> registers
+    uint32_t rda[NRA], rdb[NRB];
+    RA::template read_offsets<WM>(rda, WM * wm, lane);
+    RB::template read_offsets<WN>(rdb, WN * wn, lane);
 
     f32x16 acc[WN][WM];   // [n tile][m tile]
 #pragma unroll
@@ -140,63 +206,49 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-    const int steps0 = (klen0 + BK - 1) / BK;
-    const int steps1 = pr.nseg > 1 ? (pr.K[1] + BK - 1) / BK : 0;
-    const int steps = steps0 + steps1;
-
-    TileLoader<A_MCONTIG, TM> la;
-    TileLoader<B_NCONTIG, TN> lb;
-    const char* abase = nullptr;
-    const char* bbase = nullptr;
-    int64_t a_kstride = 0, b_kstride = 0;   // bytes per 64 k
-    int seg_len = 0, seg_first = 0;
-    auto enter_segment = [&](int seg) {
-        const int64_t lda = pr.lda[seg], ldb = pr.ldb[seg];
-        la.setup(lda, m0, p.M_ld, tid, p.a_tiled_m);
-        lb.setup(ldb, n0, p.N, tid, 0);
-        abase = reinterpret_cast<const char*>(pr.A[seg] + a_off);
-        if (!p.a_tiled_m) abase += (A_MCONTIG ? (int64_t)m0 : (int64_t)m0 * lda) * 2;
-        bbase = reinterpret_cast<const char*>(pr.Bm[seg] + b_off) + (B_NCONTIG ? (int64_t)n0 : (int64_t)n0 * ldb) * 2;
-        a_kstride = A_MCONTIG ? (p.a_tiled_m ? 0 : lda * BK * 2) : BK * 2;
-        b_kstride = B_NCONTIG ? ldb * BK * 2 : BK * 2;
-        seg_len = seg ? pr.K[1] : klen0;
-        seg_first = seg ? steps0 : 0;
-    };
-    // issue the loads of stage s; returns K - k0 of that stage
-    auto prefetch = [&](int s) {
-        if (s == 0 && steps0 > 0) enter_segment(0);
-        else if (s == steps0) enter_segment(1);
-        const int ks = s - seg_first;
-        const int krem = seg_len - ks * BK;
-        const char* ab = abase + ks * a_kstride;
-        if (A_MCONTIG && p.a_tiled_m)   // tile row of 128 k: [k / 128][m / 32][128][32]
-            ab = abase + ((int64_t)(ks >> 1) * p.a_tiled_m * 4096 + (ks & 1) * 2048) * 2;
-        la.load(ab, krem, tid);
-        lb.load(bbase + ks * b_kstride, krem, tid);
-        return krem;
-    };
-    int krem = BK;
-    if (steps > 0) krem = prefetch(0);
+    // prologue: stages 0 .. NS-2 in flight, stage 0 landed
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s)
+        if (s < steps) issue(s);
+    if (steps > NS - 2) wait_vmcnt<(NS - 2) * LPG>();
+    else wait_vmcnt<0>();
+    phase_barrier();
+    if (set == 1) phase_barrier();        // waves 4-7 run half a stage behind waves 0-3
 
     for (int s = 0; s < steps; ++s) {
-        __syncthreads();
-        la.store(As, krem, tid);
-        lb.store(Bs, krem, tid);
-        __syncthreads();
-        if (s + 1 < steps) krem = prefetch(s + 1);
+        // memory phase: request stage s+NS-1, fetch this wave's operands of stage s
+        if (s + NS - 1 < steps) issue(s + NS - 1);
+        const uint32_t base = (uint32_t)(s % NS) * STAGE;
+        bf16x8 am[2][WM], bn[2][WN];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            bf16x8 am[WM], bn[WN];
+        for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-            for (int t = 0; t < WM; ++t) am[t] = tile_operand<A_MCONTIG, TM>(As, 32 * (WM * wm + t), kk, lane, tr_off_a);
+            for (int t = 0; t < WM; ++t) am[kk][t] = RA::operand(lds, base, rda, t, kk);
 #pragma unroll
-            for (int t = 0; t < WN; ++t) bn[t] = tile_operand<B_NCONTIG, TN>(Bs, 32 * (WN * wn + t), kk, lane, tr_off_b);
+            for (int t = 0; t < WN; ++t) bn[kk][t] = RB::operand(lds, base + RA::BYTES, rdb, t, kk);
+        }
+        wait_lds();     // the slot may be overwritten once the next barrier is passed
+        if (set == 1) {                     // stage s+1 must have landed before waves 0-3 read it
+            if (s + NS - 1 < steps) wait_vmcnt<(NS - 2) * LPG>();
+            else wait_vmcnt<0>();
+        }
+        phase_barrier();
+        // compute phase
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
             for (int nt = 0; nt < WN; ++nt)
 #pragma unroll
-                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = mfma32(bn[nt], am[mt], acc[nt][mt]);
+                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = mfma32(bn[kk][nt], am[kk][mt], acc[nt][mt]);
+        __builtin_amdgcn_s_setprio(0);
+        if (set == 0) {
+            if (s + NS - 1 < steps) wait_vmcnt<(NS - 2) * LPG>();
+            else wait_vmcnt<0>();
         }
+        phase_barrier();
     }
+    if (set == 0) phase_barrier();
 
     // C^T tile: accumulator rows = n, cols = m
 #pragma unroll
@@ -218,19 +270,38 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const GemmParams p) {
     }
 }
 
-}  // namespace
-
-hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+template <int GM, int GN, int WM, int WN, int NS>
+hipError_t launch_cfg(GemmParams p, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+    constexpr int TM = 32 * WM * GM, TN = 32 * WN * GN;
+    p.tiles_m = (p.M + TM - 1) / TM;
+    p.tiles_n = (p.N + TN - 1) / TN;
+    p.total_wg = p.nprob * p.nbatch * p.tiles_m * p.tiles_n;
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (!a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, false, GEMM_WM, GEMM_WN>), dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((gemm_kernel<false, false, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
     else if (!a_mcontig && b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, true, GEMM_WM, GEMM_WN>), dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((gemm_kernel<false, true, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
     else if (a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<true, false, GEMM_WM, GEMM_WN>), dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((gemm_kernel<true, false, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
     else
-        hipLaunchKernelGGL((gemm_kernel<true, true, GEMM_WM, GEMM_WN>), dim3(grid), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((gemm_kernel<true, true, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
     return hipGetLastError();
+}
+
+}  // namespace
+
+// Work-group tile by shape: 256 x 256 in general; for a narrow C (N <= 128, the
+// dQ GEMM) 512 x 128, or 256 x 128 when there are not 512 rows.
+hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+    for (int i = 0; i < p.nprob; ++i) {
+        const GemmProblem& pr = p.prob[i];
+        // all problems and both contraction segments share the per-thread load offsets
+        if (pr.lda[0] != p.prob[0].lda[0] || pr.ldb[0] != p.prob[0].ldb[0]) return hipErrorInvalidValue;
+        if (pr.nseg > 1 && (pr.lda[1] != pr.lda[0] || pr.ldb[1] != pr.ldb[0])) return hipErrorInvalidValue;
+    }
+    if (p.N > 128) return launch_cfg<2, 4, 4, 2, 4>(p, a_mcontig, b_ncontig, st);
+    if (p.M > 256) return launch_cfg<8, 1, 2, 4, 3>(p, a_mcontig, b_ncontig, st);
+    return launch_cfg<4, 2, 2, 2, 4>(p, a_mcontig, b_ncontig, st);
 }
 
 }  // namespace lvx

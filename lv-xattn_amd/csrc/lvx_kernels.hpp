@@ -91,15 +91,6 @@ struct CastParams {
     int B, H, L;
 };
 
-// MFMA tiles (32 x 32) per wave along M and N; a work-group is 2 x 2 waves,
-// so its tile of C is (64 GEMM_WM) x (64 GEMM_WN).
-#ifndef GEMM_WM
-#define GEMM_WM 4
-#endif
-#ifndef GEMM_WN
-#define GEMM_WN 2
-#endif
-
 // One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].
 struct GemmProblem {
     const uint16_t* A[2];
@@ -121,7 +112,7 @@ struct GemmParams {
     int nprob;
     int M, N;
     int M_ld;                  // rows of A that may be loaded (>= M; rows in [M, M_ld) are padding)
-    int tiles_m, tiles_n, total_wg;
+    int tiles_m, tiles_n, total_wg;   // filled in by launch_gemm for the tile it picks
     int nbatch, batch_inner, b_group;
     int64_t a_batch, b_outer, b_inner, c_outer, c_inner;
     const int32_t* k_len;
