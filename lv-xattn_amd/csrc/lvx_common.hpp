@@ -102,6 +102,36 @@ __device__ __forceinline__ bf16x8 lds_operand_tr(const uint16_t* p, int half_off
     return as_bf16x8(u);
 }
 
+// 64 lanes x 16 bytes from global memory to the 1 KiB of LDS at byte address
+// lds_byte (wave-uniform); lane i lands at lds_byte + 16 i.  Counted by vmcnt.
+__device__ __forceinline__ void dma16(const char* sbase, uint32_t voff, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_addr(const char* addr, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte), "v"(addr) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// max of three (one instruction; fmaxf chains cost an extra canonicalising
+// v_max per MFMA result)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// acc + lo + hi of a packed bf16 pair (v_dot2c_f32_bf16 with (1, 1))
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ float sum2_bf16(uint32_t pair, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), __builtin_bit_cast(bf16x2_t, 0x3f803f80u),
+                                           acc, false);
+}
+
 // Work-groups are dealt to the 8 XCDs round-robin by linear id.  Remap so that
 // each XCD receives one contiguous range of the work list: neighbours in the
 // list (which share K/V or Q tiles) then share that XCD's L2.

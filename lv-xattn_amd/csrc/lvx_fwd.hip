@@ -18,14 +18,16 @@
 //                    row-major V tile with the transposing LDS read, addressed
 //                    in that same key order, so P never visits LDS and V is
 //                    never transposed in memory)
-// K and V are both staged row-major: K [64][128+8] (68-dword rows: the 16-byte
-// operand reads of 16 consecutive lanes hit 64 distinct banks), V [64][128+16]
-// (72-dword rows: the 8 rows x 16 dwords a transposing read touches tile the
-// banks twice).  The LDS tiles are double-buffered: while tile t is consumed,
-// tile t+1 moves from registers into the other buffer and tile t+2's global
-// loads are issued, with one barrier per tile.  Loads past the end of the key
-// range are clamped to its last row (those keys are masked out of S), so the
-// loop body has no divergent branch.
+// K and V tiles ([64 keys][128] bf16, 16 KiB each) go from global memory
+// straight into LDS with global_load_lds_dwordx4, double-buffered: tile t+1 is
+// in flight while tile t is consumed, one barrier per tile, no staging
+// registers and no LDS stores.  That load writes 64 lanes x 16 bytes
+// contiguously, so rows cannot be padded; instead the 16-byte chunk c of row r
+// is kept at position c ^ f(r), f(r) = ((r & 3) << 2) | ((r >> 2) & 3): the 16
+// rows a 16-byte operand read of K touches land in 16 different positions, and
+// the 4 rows a transposing read of V touches land in 4 different 64-byte
+// groups - both conflict-free.  Loads past the end of the key range are
+// clamped to its last row (those keys are masked out of S).
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -35,14 +37,12 @@ namespace {
 
 constexpr int D = 128;
 constexpr int BN = 64;        // keys per tile
-constexpr int KS = D + 8;     // K tile row stride (elements)
-constexpr int VS = D + 16;    // V tile row stride (elements)
+constexpr int TILE_BYTES = BN * D * 2;
 constexpr int BIG = 0x3fffffff;
 
 template <bool MASKED>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs2[2][BN * VS];
+    __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     const int b = t2 / p.n_head_groups;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int h = hg * p.HG + (wave % p.HG);
     const int hk = h / p.G;
     const int row = p.row_begin + (tile * p.RS + wave / p.HG) * 32 + l32;
@@ -97,6 +97,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         in_lo = max(in_lo, red[w][2]);
         in_hi = min(in_hi, red[w][3]);
     }
+    // the same in every lane of the work-group: keep them in scalar registers
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    in_lo = __builtin_amdgcn_readfirstlane(in_lo);
+    in_hi = __builtin_amdgcn_readfirstlane(in_hi);
 
     // Q^T as B operand, resident for the whole kernel
     bf16x8 qreg[8];
@@ -106,27 +111,44 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int kk = 0; kk < 8; ++kk) qreg[kk] = as_bf16x8(ldg16(qp + kk * 16, row_ok));
     }
 
-    const uint16_t* kbase = p.k + b * p.ks.b + hk * p.ks.h;
-    const uint16_t* vbase = p.v + b * p.vs.b + hk * p.vs.h;
-    const int off_vT = tr_lane_offset(lane, VS, true);   // V^T operand, keys in accumulator order
+    const char* kbase = reinterpret_cast<const char*>(p.k + b * p.ks.b + hk * p.ks.h);
+    const char* vbase = reinterpret_cast<const char*>(p.v + b * p.vs.b + hk * p.vs.h);
+    const uint32_t krow_b = (uint32_t)p.ks.s * 2u, vrow_b = (uint32_t)p.vs.s * 2u;   // bytes per key row
 
-    u32x4 kpre[4], vpre[4];
-    const int ld_row = tid >> 4, ld_col = (tid & 15) * 8;   // this thread's chunk of rows ld_row + 16 i
-    auto prefetch = [&](int kv0) {
+    // global -> LDS: wave w moves the 1 KiB chunks w, w+4, w+8, w+12 (4 rows each)
+    // of the K tile and of the V tile; lane i fills position i & 15 of row i >> 4.
+    const int wave_u = wave;
+    const int ld_r = lane >> 4;
+    const uint32_t ld_c = (uint32_t)((lane & 15) ^ ((ld_r << 2) | wave_u)) * 16u;   // chunk this lane fetches
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&kv_lds[0][0][0];
+    auto issue = [&](int kv0, int buf) {
+        const char* kb = kbase + (int64_t)kv0 * krow_b;
+        const char* vb = vbase + (int64_t)kv0 * vrow_b;
+        const uint32_t slot = lds0 + (uint32_t)buf * (2 * TILE_BYTES) + (uint32_t)wave_u * 1024u;
+        const int last = kv_hi - 1 - kv0;          // rows past `last` repeat it
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int kv = min(kv0 + ld_row + 16 * i, kv_hi - 1);
-            kpre[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kv * p.ks.s + ld_col);
-            vpre[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kv * p.vs.s + ld_col);
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = (uint32_t)min(4 * (wave_u + 4 * j) + ld_r, last);
+            dma16(kb, r * krow_b + ld_c, slot + j * 4096);
+            dma16(vb, r * vrow_b + ld_c, slot + TILE_BYTES + j * 4096);
         }
     };
-    auto stage = [&](int buf) {
+
+    // LDS -> operands.  K rows (A of S^T): 16 bytes at row * 256 + ((2 kk + g) ^ f(row)) * 16.
+    const int f_row = ((l32 & 3) << 2) | ((l32 >> 2) & 3);
+    const uint32_t k_rd = (uint32_t)(l32 * 256), k_h = (uint32_t)((g ^ f_row) << 4);
+    // V^T (A of O^T += V^T P^T), keys in accumulator order: first half rows 16 j + 4 g + r,
+    // second half 8 rows further down, whose f differs in bit 1.
+    uint32_t v_rd[4][2];
+    {
+        const int r = (lane & 15) >> 2, t = lane & 3, u = (lane >> 4) & 1;
+        const int low = (2 * u + (t >> 1)) ^ g;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4*>(&Ks2[buf][(ld_row + 16 * i) * KS + ld_col]) = kpre[i];
-            *reinterpret_cast<u32x4*>(&Vs2[buf][(ld_row + 16 * i) * VS + ld_col]) = vpre[i];
+        for (int dt = 0; dt < 4; ++dt) {
+            v_rd[dt][0] = (uint32_t)((4 * g + r) * 256 + (4 * (dt ^ r) + low) * 16 + (t & 1) * 8);
+            v_rd[dt][1] = (uint32_t)((4 * g + r + 8) * 256 + (4 * (dt ^ r) + (low ^ 2)) * 16 + (t & 1) * 8);
         }
-    };
+    }
 
     f32x16 acc[4];
 #pragma unroll
@@ -138,18 +160,20 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
     const int t_begin = (hi > lo) ? lo / BN : 0;
     const int t_end = (hi > lo) ? (hi + BN - 1) / BN : 0;
-    if (t_end > t_begin) {
-        prefetch(t_begin * BN);
-        stage(0);
-        __syncthreads();
-        prefetch(min(t_begin + 1, t_end - 1) * BN);
-    }
+    if (t_end > t_begin) issue(t_begin * BN, 0);
 
     for (int t = t_begin; t < t_end; ++t) {
         const int kv0 = t * BN;
         const int buf = (t - t_begin) & 1;
-        const uint16_t* Ks = Ks2[buf];
-        const uint16_t* Vs = Vs2[buf];
+        const char* Ks = kv_lds[buf][0];
+        const char* Vs = kv_lds[buf][1];
+
+        // tile t has landed (this wave's part: vmcnt; everyone's: barrier); the
+        // barrier also says every wave is done reading tile t-1, whose buffer
+        // the loads of tile t+1 may now overwrite
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (t + 1 < t_end) issue(kv0 + BN, buf ^ 1);
 
         // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows
         f32x16 s0, s1;
@@ -157,8 +181,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-            const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(&Ks[l32 * KS + kk * 16 + g * 8]);
-            const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(&Ks[(32 + l32) * KS + kk * 16 + g * 8]);
+            const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+            const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(kp);
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
             s0 = mfma32(a0, qreg[kk], s0);
             s1 = mfma32(a1, qreg[kk], s1);
         }
@@ -172,40 +197,39 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
             }
         }
 
-        float mx = fmaxf(s0[0], s1[0]);
+        float mx = max3(s0[0], s1[0], s0[1]);
+        mx = max3(mx, s1[1], s0[2]);
 #pragma unroll
-        for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(s0[v], s1[v]));
+        for (int v = 3; v < 16; v += 1) mx = max3(mx, s1[v - 1], s0[v]);
+        mx = fmaxf(mx, s1[15]);
         {   // other half of the wave holds the other 32 keys of the same text row
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+            mx = max3(__uint_as_float(sw[0]), __uint_as_float(sw[1]), m_i);
         }
-        const float m_new = fmaxf(m_i, mx);
+        const float m_new = mx;
         const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
         const float alpha = __builtin_amdgcn_exp2f(m_i * c - mc);
         m_i = m_new;
 
-        float rs = 0.f;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            s0[v] = __builtin_amdgcn_exp2f(fmaf(s0[v], c, -mc));
-            s1[v] = __builtin_amdgcn_exp2f(fmaf(s1[v], c, -mc));
-            rs += s0[v] + s1[v];
-        }
-        l_i = l_i * alpha + rs;
-
-        // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile
+        // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile; the row
+        // sum is taken over the bf16-rounded P, the values the MFMA sees
         bf16x8 pb[4];
+        float rs0 = 0.f, rs1 = 0.f;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             u32x4 u0, u1;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                u0[e] = pack_bf16(s0[8 * j + 2 * e], s0[8 * j + 2 * e + 1]);
-                u1[e] = pack_bf16(s1[8 * j + 2 * e], s1[8 * j + 2 * e + 1]);
+                const int v = 8 * j + 2 * e;
+                u0[e] = pack_bf16(__builtin_amdgcn_exp2f(fmaf(s0[v], c, -mc)), __builtin_amdgcn_exp2f(fmaf(s0[v + 1], c, -mc)));
+                u1[e] = pack_bf16(__builtin_amdgcn_exp2f(fmaf(s1[v], c, -mc)), __builtin_amdgcn_exp2f(fmaf(s1[v + 1], c, -mc)));
+                rs0 = sum2_bf16(u0[e], rs0);
+                rs1 = sum2_bf16(u1[e], rs1);
             }
             pb[j] = as_bf16x8(u0);
             pb[2 + j] = as_bf16x8(u1);
         }
+        l_i = l_i * alpha + (rs0 + rs1);
 
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {   // the running max moved for some row
 #pragma unroll
@@ -219,17 +243,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const bf16x8 a = lds_operand_tr(&Vs[off_vT + 16 * j * VS + dt * 32], 8 * VS);
-                acc[dt] = mfma32(a, pb[j], acc[dt]);
+                const u32x2 lo2 = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
+                const u32x2 hi2 = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][1] + j * 4096));
+                const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                acc[dt] = mfma32(as_bf16x8(a), pb[j], acc[dt]);
             }
-
-        // tile t+1 (in registers since the previous iteration) goes to the other
-        // buffer, whose last readers finished before the previous barrier
-        if (t + 1 < t_end) {
-            stage(buf ^ 1);
-            __syncthreads();
-            prefetch(min(t + 2, t_end - 1) * BN);
-        }
     }
 
     // epilogue: the two lane halves hold partial row sums of the same row

@@ -32,20 +32,6 @@ namespace {
 constexpr int BK = 32;                 // contraction depth of one stage
 __device__ uint32_t zero_chunk[4];     // source of the chunks past the end of a contraction
 
-// 64 lanes x 16 bytes from global memory to the 1 KiB of LDS at byte address
-// lds_byte (wave-uniform); lane i lands at lds_byte + 16 i.  Counted by vmcnt.
-__device__ __forceinline__ void dma16(const char* sbase, uint32_t voff, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte), "v"(voff), "s"(sbase)
-                 : "memory", "m0");
-}
-__device__ __forceinline__ void dma16_addr(const char* addr, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte), "v"(addr) : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
