@@ -125,13 +125,6 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return r;
 }
 
-// acc + lo + hi of a packed bf16 pair (v_dot2c_f32_bf16 with (1, 1))
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-__device__ __forceinline__ float sum2_bf16(uint32_t pair, float acc) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), __builtin_bit_cast(bf16x2_t, 0x3f803f80u),
-                                           acc, false);
-}
-
 // Work-groups are dealt to the 8 XCDs round-robin by linear id.  Remap so that
 // each XCD receives one contiguous range of the work list: neighbours in the
 // list (which share K/V or Q tiles) then share that XCD's L2.

@@ -39,6 +39,7 @@ constexpr int D = 128;
 constexpr int BN = 64;        // keys per tile
 constexpr int TILE_BYTES = BN * D * 2;
 constexpr int BIG = 0x3fffffff;
+constexpr float RESCALE_LOG2 = 8.f;
 
 template <bool MASKED>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
@@ -175,18 +176,36 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         __syncthreads();
         if (t + 1 < t_end) issue(kv0 + BN, buf ^ 1);
 
-        // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows
+        // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows.
+        // All 16 K operands are requested before the first MFMA, so the LDS
+        // latency is paid once per tile and not once per k-step.
+        bf16x8 ka[8][2];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+            ka[kk][0] = *reinterpret_cast<const bf16x8*>(kp);
+            ka[kk][1] = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         f32x16 s0, s1;
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-            const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
-            const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(kp);
-            const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
-            s0 = mfma32(a0, qreg[kk], s0);
-            s1 = mfma32(a1, qreg[kk], s1);
+            s0 = mfma32(ka[kk][0], qreg[kk], s0);
+            s1 = mfma32(ka[kk][1], qreg[kk], s1);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        // V^T operands of this tile: requested now, they land during the softmax
+        u32x2 va[4][4][2];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                va[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
+                va[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][1] + j * 4096));
+            }
+        __builtin_amdgcn_sched_barrier(0);
 
         if (kv0 < in_lo || kv0 + BN > in_hi) {
 #pragma unroll
@@ -206,13 +225,20 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
             mx = max3(__uint_as_float(sw[0]), __uint_as_float(sw[1]), m_i);
         }
-        const float m_new = mx;
-        const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
-        const float alpha = __builtin_amdgcn_exp2f(m_i * c - mc);
-        m_i = m_new;
+        // Lazy rescale: the reference point m_i of a row only moves when the row
+        // maximum has grown by more than 2^RESCALE_LOG2 since it was set, so P may
+        // reach 2^RESCALE_LOG2 instead of 1 (harmless in fp32 / bf16) and the
+        // rescale of O happens a few times per row instead of almost every tile.
+        const float mcand = mx * c;                       // mx >= m_i
+        const float m_ic = m_i * c;
+        const bool move = (mx != -INFINITY) && !(mcand - m_ic <= RESCALE_LOG2);
+        const float alpha = move ? __builtin_amdgcn_exp2f(m_ic - mcand) : 1.f;
+        if (move) m_i = mx;
+        const float mc = (m_i == -INFINITY) ? 0.f : m_i * c;
 
-        // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile; the row
-        // sum is taken over the bf16-rounded P, the values the MFMA sees
+        // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile.  The row
+        // sum is taken in fp32 before the rounding to bf16 (summing the rounded
+        // values would put the LSE off by up to a bf16 ulp of the largest term).
         bf16x8 pb[4];
         float rs0 = 0.f, rs1 = 0.f;
 #pragma unroll
@@ -221,10 +247,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int v = 8 * j + 2 * e;
-                u0[e] = pack_bf16(__builtin_amdgcn_exp2f(fmaf(s0[v], c, -mc)), __builtin_amdgcn_exp2f(fmaf(s0[v + 1], c, -mc)));
-                u1[e] = pack_bf16(__builtin_amdgcn_exp2f(fmaf(s1[v], c, -mc)), __builtin_amdgcn_exp2f(fmaf(s1[v + 1], c, -mc)));
-                rs0 = sum2_bf16(u0[e], rs0);
-                rs1 = sum2_bf16(u1[e], rs1);
+                const float a0 = __builtin_amdgcn_exp2f(fmaf(s0[v], c, -mc)), a1 = __builtin_amdgcn_exp2f(fmaf(s0[v + 1], c, -mc));
+                const float b0 = __builtin_amdgcn_exp2f(fmaf(s1[v], c, -mc)), b1 = __builtin_amdgcn_exp2f(fmaf(s1[v + 1], c, -mc));
+                rs0 += a0 + a1;
+                rs1 += b0 + b1;
+                u0[e] = pack_bf16(a0, a1);
+                u1[e] = pack_bf16(b0, b1);
             }
             pb[j] = as_bf16x8(u0);
             pb[2 + j] = as_bf16x8(u1);
@@ -239,13 +267,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         }
 
         // O^T += V^T P^T
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32x2 lo2 = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
-                const u32x2 hi2 = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][1] + j * 4096));
-                const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                const u32x4 a = {va[dt][j][0][0], va[dt][j][0][1], va[dt][j][1][0], va[dt][j][1][1]};
                 acc[dt] = mfma32(as_bf16x8(a), pb[j], acc[dt]);
             }
     }
