@@ -152,6 +152,45 @@ def kernel_breakdown(layer, n_pairs, torch):
     return res
 
 
+def run_only(layer, which, n, torch):
+    """`n` launches of one operator at the workload's full size, nothing else on
+    the GPU afterwards: the target of the rocprofv3 --pmc runs."""
+    ops, w = layer.ops, layer.w
+    dev = layer.q.device
+    if which == "copy":
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(n):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"only": which, "launches": n, "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
+    k, v = layer.project()
+    B, Hq, Lq, D = layer.q.shape
+    Hkv, Lkv = k.shape[1], k.shape[2]
+    o, L = torch.empty_like(layer.q), torch.empty(B * Hq, Lq, device=dev)
+    ops.fwd(layer.q, k, v, o, L, w.scale, mask=layer.mask)
+    if which == "fwd":
+        fn = lambda: ops.fwd(layer.q, k, v, o, L, w.scale, mask=layer.mask)
+    elif which == "bwd":
+        delta = torch.empty_like(L)
+        ops.bwd_preprocess(o, layer.do, delta)
+        dq = torch.empty_like(layer.q)
+        bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq), dtype=torch.uint8, device=dev)
+        dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+        dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
+        fn = lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask, workspace=bws)
+    elif which == "kv_proj":
+        fn = layer.project
+    else:
+        fn = lambda: ops.dx_vis(k, v, layer.wk, layer.wv)
+    torch.cuda.synchronize()
+    for _ in range(n):
+        fn()
+    torch.cuda.synchronize()
+    print(json.dumps({"only": which, "launches": n, "workload": w.name}))
+
+
 def cpu_baseline(w, budget_rounds=2):
     """The oracle (the reference's PyTorch math restated) timed on this host's
     cores on a bounded sample: the first `budget_rounds` query blocks, forward
@@ -203,6 +242,9 @@ def main():
     ap.add_argument("--mode", default="batched", choices=["batched", "rounds"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--only", choices=["fwd", "bwd", "kv_proj", "dx_vis", "copy"],
+                    help="launch just this operator --steps times (for rocprofv3 counter runs); "
+                         "'copy' is a 1 GiB device copy that calibrates FETCH_SIZE / WRITE_SIZE")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build is a single-GPU path (no collectives, no sharding); run with --gpus 1")
@@ -220,6 +262,9 @@ def main():
     step_flops = f["fwd"] + f["bwd"] + 3 * f["proj"]    # projection, re-projection, dX_vis
 
     layer = Layer(w, a.mode, dev)
+    if a.only:
+        run_only(layer, a.only, a.steps, torch)
+        return
     for _ in range(a.warmup):
         layer.step()
     torch.cuda.synchronize()
