@@ -25,6 +25,9 @@ for p in (ROOT, os.path.join(ROOT, "lv-xattn_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes moved by one lvx_bwd call at cfg2 (zero + dK/dV kernel + 2 casts + dQ GEMM), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy (profiles/cfg2_bwd_hbm_traffic.md)
+BWD_TRAFFIC_BYTES = {"cfg2": 4.41e9}
 
 
 def flops(w, n_pairs):
@@ -191,7 +194,7 @@ def run_only(layer, which, n, torch):
     print(json.dumps({"only": which, "launches": n, "workload": w.name}))
 
 
-def cpu_baseline(w, budget_rounds=2):
+def cpu_baseline(w, budget_rounds=8):
     """The oracle (the reference's PyTorch math restated) timed on this host's
     cores on a bounded sample: the first `budget_rounds` query blocks, forward
     + backward against the full shard, plus the K/V projection twice and
@@ -292,16 +295,17 @@ def main():
         kb = kernel_breakdown(layer, npairs, torch)
         out["kernels"] = kb
         dom = kb["bwd_all_rounds_one_launch"]
-        out["roofline"] = {"bound": "mfma", "kernel": "bwd_kernel<false>", "achieved": dom["tflops"],
-                           "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                           "avg_launch_ms": dom["ms"]}
+        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = zero_kernel + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
+                           "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                           "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
+                           "traffic": BWD_TRAFFIC_BYTES.get(w.name) if a.mode == "batched" else None,
+                           "flops_per_launch": f["bwd"], "avg_launch_ms": dom["ms"]}
         other = Layer(w, "rounds" if a.mode == "batched" else "batched", dev)
         ms2 = time_gpu(other.step, max(3, a.steps // 2), 2, torch)
         out["config"]["other_mode"] = {"mode": other.mode, "ms_per_step": round(ms2, 4),
                                        "tflops": round(step_flops / ms2 / 1e9, 2)}
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"] = cpu_baseline(w, min(8, w.rounds))
     print(json.dumps(out))
 
 
