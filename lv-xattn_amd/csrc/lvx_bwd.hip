@@ -25,11 +25,17 @@
 // batched GEMM (launched by the caller right after) contracts it with K.  The workspace costs 2 bytes per (row, token, head),
 // written once and read once.
 //
-// All MFMA are 32x32x16 bf16.  A operands come from LDS: Q / dO rows by 16-byte
-// reads, Q^T / dO^T by the transposing LDS read of a second copy of the same
-// row-major tile (no single row stride is conflict-free for both patterns), the
-// latter addressed in the accumulator's row order so that P / dS go from the
-// registers straight into the next MFMA as B operands.
+// All MFMA are 32x32x16 bf16.  A operands come from LDS.  The Q and dO tiles
+// ([32 rows][128] bf16, 8 KiB each) go from global memory straight into LDS
+// with global_load_lds_dwordx4, two steps ahead, into a ring of four buffers;
+// the load writes 64 lanes x 16 bytes contiguously, so rows are not padded:
+// the 16-byte chunk c of row r is kept at position c ^ f(r),
+// f(r) = ((r & 3) << 2) | ((r >> 2) & 3), which makes both access patterns
+// conflict-free on ONE copy of a tile - Q / dO rows by 16-byte reads, Q^T /
+// dO^T by the transposing LDS read, the latter addressed in the accumulator's
+// row order so that P / dS go from the registers straight into the next MFMA
+// as B operands.  Every wave requests all LDS operands of a step before its
+// first MFMA, so their latency is paid once per step.
 #include <type_traits>
 
 #include "lvx_common.hpp"
@@ -43,20 +49,16 @@ constexpr int D = 128;
 constexpr int BN = 128;       // visual tokens per work-group
 constexpr int BM = 32;        // text rows per step
 constexpr int NT = 512;       // threads per work-group
-constexpr int QS = D + 8;     // row stride of the tile copies read by rows       (68 dwords)
-constexpr int QT = D + 16;    // row stride of the tile copies read transposed    (72 dwords)
 constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row]
 
-// one staged (Q, dO) tile set: Q rows | dO rows | Q for transposed reads | dO for transposed reads
-constexpr int OFF_QR = 0;
-constexpr int OFF_DOR = OFF_QR + BM * QS;
-constexpr int OFF_QTR = OFF_DOR + BM * QS;
-constexpr int OFF_DOTR = OFF_QTR + BM * QT;
-constexpr int QD_ELEMS = OFF_DOTR + BM * QT;
+// LDS map (uint16 units): four (Q | dO) tile pairs, unpadded; two dS^T tiles; two P hand-over buffers
+constexpr int TILE_ELEMS = BM * D;             // one Q or dO tile (8 KiB)
+constexpr int QD_ELEMS = 2 * TILE_ELEMS;
+constexpr int NQD = 4;
 constexpr int DST_ELEMS = BN * DSS;
 constexpr int PB_ELEMS = 4 * 2 * 64 * 8;       // P hand-over: [slice][half][lane][16 bytes] as uint16
-constexpr int OFF_QD = 0;                      // x3
-constexpr int OFF_DST = OFF_QD + 3 * QD_ELEMS; // x2
+constexpr int OFF_QD = 0;                      // x4
+constexpr int OFF_DST = OFF_QD + NQD * QD_ELEMS; // x2
 constexpr int OFF_PB = OFF_DST + 2 * DST_ELEMS;  // x2
 constexpr int LOOP_ELEMS = OFF_PB + 2 * PB_ELEMS;
 constexpr int EPS = D + 1;                          // row stride (floats) of the epilogue's transposed tile
@@ -67,7 +69,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 template <bool MASKED>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t smem[SMEM_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
     // per-row metadata of a staged tile, triple-buffered: 8 x 16 bytes each of
     // LSE*log2e, delta, kv_start, kv_end
     __shared__ u32x4 meta_s4[3][BM];
@@ -114,16 +116,12 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const int n_iter = (kvb < kv_len) ? max(0, min(p.split_steps, p.G * n_qtiles - it_lo)) : 0;
     const float c = p.scale_log2e;
 
-    // staging role of this thread: threads 0..255 carry Q, 256..511 carry dO; two
-    // 16-byte chunks each (rows s_row and s_row + 16)
-    const int st = tid & 255;
-    const int s_row = st >> 4, s_chunk = st & 15;
-    const bool is_do = tid >= 256;
-    const int stage_off = (is_do ? OFF_DOR : OFF_QR) + s_row * QS + s_chunk * 8;
-    const int stage_off_t = (is_do ? OFF_DOTR : OFF_QTR) + s_row * QT + s_chunk * 8;
-    const uint16_t* g_base = is_do ? p.dout + b * p.dos.b : p.q + b * p.qs.b;
-    const int64_t g_hs = is_do ? p.dos.h : p.qs.h;
-    const int g_rs = (int)(is_do ? p.dos.s : p.qs.s);
+    // global -> LDS: wave w moves rows 4w..4w+3 of the Q tile and of the dO tile
+    // (one 1 KiB load each); lane i fills position i & 15 of row 4w + (i >> 4).
+    const int ld_r = 4 * wave + (lane >> 4);
+    const uint32_t ld_c = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | (wave & 3))) * 16u;
+    const uint32_t qrow_b = (uint32_t)p.qs.s * 2u, dorow_b = (uint32_t)p.dos.s * 2u;   // bytes per text row
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const int meta_kind = (tid >> 5) & 3;    // 0 LSE, 1 delta, 2 kv_start, 3 kv_end (threads 0..127)
     const uint32_t* m_base = reinterpret_cast<const uint32_t*>(p.lse);
     int64_t m_hs = p.Lq;
@@ -137,7 +135,21 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     // per-lane offsets: transposing operand reads (rows in accumulator order),
     // P hand-over slot, dS^T copy-out (512 chunks of 16 bytes, one per thread)
-    const int off_tr = tr_lane_offset(lane, QT, true);
+    // rows: 16 bytes at row * 256 + ((2 kk + g) ^ f(row)) * 16
+    const uint32_t row_rd = (uint32_t)(l32 * 256);
+    const uint32_t row_h = (uint32_t)((g ^ (((l32 & 3) << 2) | ((l32 >> 2) & 3))) << 4);
+    // transposed, rows in accumulator order: first half rows 16 j + 4 g + r, second
+    // half 8 rows further down (its f differs in bit 1); add j * 4096
+    uint32_t t_rd[4][2];
+    {
+        const int r = (lane & 15) >> 2, t = lane & 3, u = (lane >> 4) & 1;
+        const int low = (2 * u + (t >> 1)) ^ g;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            t_rd[dt][0] = (uint32_t)((4 * g + r) * 256 + (4 * (dt ^ r) + low) * 16 + (t & 1) * 8);
+            t_rd[dt][1] = (uint32_t)((4 * g + r + 8) * 256 + (4 * (dt ^ r) + (low ^ 2)) * 16 + (t & 1) * 8);
+        }
+    }
     const int pb_off = slice * (2 * 64 * 8) + lane * 8;
     const int cp_token = tid >> 2, cp_part = tid & 3;
     // workspace tile (b, h, token block, row tile): [128 tokens][32 rows], 8 KB, contiguous
@@ -148,24 +160,21 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // Every load is unconditional: rows past the window are clamped to its last
     // row (their LSE is forced to +inf, so P = 0 and nothing they carry reaches a
     // result), and the fetch after the last tile re-reads some tile.
-    // Two register sets alternate: the set consumed at the top of step i is
-    // refilled right after the barrier with tile i + 2, so every load has two
-    // full steps to arrive.
+    // The Q / dO tile goes straight to its LDS buffer; the row metadata travels
+    // through one of two alternating register pairs and is stored two steps later.
     struct Pre {
-        u32x4 d[2];
         uint32_t m;
         bool ok;
     };
     Pre preA{}, preB{};
-    auto prefetch = [&](Pre& pr) {
+    auto prefetch = [&](Pre& pr, int buf) {
         const int h = hk * p.G + cur_gi;
         const int r0 = p.row_begin + cur_qt * BM;
-        const uint16_t* base = g_base + h * g_hs + s_chunk * 8;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int row = min(r0 + s_row + 16 * i, p.row_end - 1);
-            pr.d[i] = *reinterpret_cast<const u32x4*>(base + row * g_rs);
-        }
+        const uint32_t row = (uint32_t)min(r0 + ld_r, p.row_end - 1);
+        const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)wave * 1024u;
+        dma16(reinterpret_cast<const char*>(p.q + b * p.qs.b + h * p.qs.h), row * qrow_b + ld_c, slot);
+        dma16(reinterpret_cast<const char*>(p.dout + b * p.dos.b + h * p.dos.h), row * dorow_b + ld_c,
+              slot + TILE_ELEMS * 2);
         const int mrow = r0 + (tid & 31);
         pr.ok = mrow < p.row_end;
         pr.m = m_base[h * m_hs + min(mrow, p.row_end - 1)];
@@ -176,12 +185,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             if (++cur_gi == p.G) cur_gi = 0;
         }
     };
-    auto stage_write = [&](const Pre& pr, uint16_t* qd, u32x4* meta) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            *reinterpret_cast<u32x4*>(qd + stage_off + 16 * i * QS) = pr.d[i];
-            *reinterpret_cast<u32x4*>(qd + stage_off_t + 16 * i * QT) = pr.d[i];
-        }
+    auto stage_write = [&](const Pre& pr, u32x4* meta) {
         const float l = __uint_as_float(pr.m);
         // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
         const float lt = (!pr.ok || l == -INFINITY) ? INFINITY : l * LOG2E;
@@ -198,13 +202,29 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // ---- P-wave: S = Q K_w^T, P = exp2(S*c - LSE*log2e) (masked), hand P over, dV_w^T += dO^T P
     auto p_step = [&](auto tail_c, const uint16_t* qd, const u32x4* meta, uint16_t* pbuf) {
         constexpr bool TAIL = decltype(tail_c)::value;
+        const char* qt = reinterpret_cast<const char*>(qd);
+        const char* dot = qt + TILE_ELEMS * 2;
+        bf16x8 qa[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            qa[kk] = *reinterpret_cast<const bf16x8*>(qt + row_rd + ((uint32_t)(kk * 32) ^ row_h));
+        __builtin_amdgcn_sched_barrier(0);
         f32x16 s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
-        const uint16_t* qrow = qd + OFF_QR + l32 * QS + g * 8;
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk)
-            s = mfma32(*reinterpret_cast<const bf16x8*>(qrow + kk * 16), breg[kk], s);
+        for (int kk = 0; kk < 8; ++kk) s = mfma32(qa[kk], breg[kk], s);
+        __builtin_amdgcn_sched_barrier(0);
+        // dO^T operands: requested now, they land during the exp2 phase
+        u32x2 da[4][2][2];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                da[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][0] + j * 4096));
+                da[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][1] + j * 4096));
+            }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int vg = 0; vg < 4; ++vg) {
             const f32x4 l4 = __builtin_bit_cast(f32x4, meta[2 * vg + g]);
@@ -233,69 +253,95 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             for (int e = 0; e < 4; ++e) pu[j][e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
         *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
         *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
-        const uint16_t* dot = qd + OFF_DOTR + off_tr;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                acc[dt] = mfma32(lds_operand_tr(dot + 16 * j * QT + dt * 32, 8 * QT), as_bf16x8(pu[j]), acc[dt]);
+            for (int j = 0; j < 2; ++j) {
+                const u32x4 a = {da[dt][j][0][0], da[dt][j][0][1], da[dt][j][1][0], da[dt][j][1][1]};
+                acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(pu[j]), acc[dt]);
+            }
     };
 
-    // ---- D-wave, first half: dP = dO V_w^T of the current tile
-    auto d_step_dp = [&](const uint16_t* qd, f32x16& dp) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) dp[v] = 0.f;
-        const uint16_t* drow = qd + OFF_DOR + l32 * QS + g * 8;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk)
-            dp = mfma32(*reinterpret_cast<const bf16x8*>(drow + kk * 16), breg[kk], dp);
-    };
-    // ---- D-wave, second half (one step later): dS = P (dP - delta) scale, dS^T to LDS, dK_w^T += Q^T dS
-    auto d_step_ds = [&](const uint16_t* qd, const u32x4* meta, const uint16_t* pbuf, uint16_t* dst,
-                         const f32x16& dp) {
+    // ---- D-wave.  For the previous tile (have_prev): dS = P (dP - delta) scale, dS^T to
+    // LDS, dK_w^T += Q^T dS; for the current tile (live): dP = dO V_w^T.  All LDS operands
+    // of both halves are requested first.
+    auto d_step = [&](bool have_prev, bool live, const uint16_t* qd_prev, const u32x4* meta, const uint16_t* pbuf,
+                      uint16_t* dst, const uint16_t* qd_cur, f32x16& dp) {
+        const char* qt = reinterpret_cast<const char*>(qd_prev);
+        const char* dor = reinterpret_cast<const char*>(qd_cur) + TILE_ELEMS * 2;
         u32x4 pu[2];
-        pu[0] = *reinterpret_cast<const u32x4*>(pbuf + pb_off);
-        pu[1] = *reinterpret_cast<const u32x4*>(pbuf + pb_off + 64 * 8);
+        u32x2 qa[4][2][2];
+        bf16x8 da[8];
+        if (have_prev) {
+            pu[0] = *reinterpret_cast<const u32x4*>(pbuf + pb_off);
+            pu[1] = *reinterpret_cast<const u32x4*>(pbuf + pb_off + 64 * 8);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    qa[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(qt + t_rd[dt][0] + j * 4096));
+                    qa[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(qt + t_rd[dt][1] + j * 4096));
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         u32x4 dsu[2];
+        if (have_prev) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const f32x4 da = __builtin_bit_cast(f32x4, meta[8 + 4 * j + g]);       // rows 16j + 4g + 0..3
-            const f32x4 db = __builtin_bit_cast(f32x4, meta[8 + 4 * j + 2 + g]);   // rows 16j + 8 + 4g + 0..3
+            for (int j = 0; j < 2; ++j) {
+                const f32x4 da4 = __builtin_bit_cast(f32x4, meta[8 + 4 * j + g]);       // rows 16j + 4g + 0..3
+                const f32x4 db4 = __builtin_bit_cast(f32x4, meta[8 + 4 * j + 2 + g]);   // rows 16j + 8 + 4g + 0..3
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // registers 8j + 2e, 8j + 2e + 1 are rows 16j + 8(e/2) + 4g + 2(e%2) + {0, 1}
-                const float d0 = (e < 2) ? da[2 * (e & 1)] : db[2 * (e & 1)];
-                const float d1 = (e < 2) ? da[2 * (e & 1) + 1] : db[2 * (e & 1) + 1];
-                const float p0 = bf16_lo(pu[j][e]) * p.scale, p1 = bf16_hi(pu[j][e]) * p.scale;
-                dsu[j][e] = pack_bf16(p0 * (dp[8 * j + 2 * e] - d0), p1 * (dp[8 * j + 2 * e + 1] - d1));
+                for (int e = 0; e < 4; ++e) {
+                    // registers 8j + 2e, 8j + 2e + 1 are rows 16j + 8(e/2) + 4g + 2(e%2) + {0, 1}
+                    const float d0 = (e < 2) ? da4[2 * (e & 1)] : db4[2 * (e & 1)];
+                    const float d1 = (e < 2) ? da4[2 * (e & 1) + 1] : db4[2 * (e & 1) + 1];
+                    const float p0 = bf16_lo(pu[j][e]) * p.scale, p1 = bf16_hi(pu[j][e]) * p.scale;
+                    dsu[j][e] = pack_bf16(p0 * (dp[8 * j + 2 * e] - d0), p1 * (dp[8 * j + 2 * e + 1] - d1));
+                }
+            }
+            uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                const u32x2 w = {dsu[vg >> 1][2 * (vg & 1)], dsu[vg >> 1][2 * (vg & 1) + 1]};
+                *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
             }
         }
-        uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
+        // dO rows of the current tile: in flight during the dK MFMAs
+        if (live) {
 #pragma unroll
-        for (int vg = 0; vg < 4; ++vg) {
-            const u32x2 w = {dsu[vg >> 1][2 * (vg & 1)], dsu[vg >> 1][2 * (vg & 1) + 1]};
-            *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
+            for (int kk = 0; kk < 8; ++kk)
+                da[kk] = *reinterpret_cast<const bf16x8*>(dor + row_rd + ((uint32_t)(kk * 32) ^ row_h));
         }
-        const uint16_t* qt = qd + OFF_QTR + off_tr;
+        __builtin_amdgcn_sched_barrier(0);
+        if (have_prev) {
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                acc[dt] = mfma32(lds_operand_tr(qt + 16 * j * QT + dt * 32, 8 * QT), as_bf16x8(dsu[j]), acc[dt]);
+                for (int j = 0; j < 2; ++j) {
+                    const u32x4 a = {qa[dt][j][0][0], qa[dt][j][0][1], qa[dt][j][1][0], qa[dt][j][1][1]};
+                    acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(dsu[j]), acc[dt]);
+                }
+        }
+        if (live) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dp[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) dp = mfma32(da[kk], breg[kk], dp);
+        }
     };
 
     auto run = [&](auto tail_c) {
         if (n_iter == 0) return;
-        // tile i lives in qd(i % 3), meta_s4[i % 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
+        // tile i lives in qd(i & 3), its row metadata in meta_s4[i % 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
         auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
         auto dst = [&](int k) { return smem + OFF_DST + k * DST_ELEMS; };
         auto pbf = [&](int k) { return smem + OFF_PB + k * PB_ELEMS; };
         // (h, r0) of the tiles: being fetched (+2, +1), current (0), previous (-1, -2)
         int h_q[5] = {0, 0, 0, 0, 0}, r_q[5] = {0, 0, 0, 0, 0};
-        auto fetch = [&](Pre& pr) {   // start the loads of the next tile of the walk
+        auto fetch = [&](Pre& pr, int buf) {   // start the loads of the next tile of the walk
             h_q[4] = hk * p.G + cur_gi;
             r_q[4] = p.row_begin + cur_qt * BM;
-            prefetch(pr);
+            prefetch(pr, buf);
             advance();
         };
         auto shift = [&]() {
@@ -309,18 +355,17 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // start tile i (dP); everyone copies dS^T(i-2) out.  Step n_iter only drains.
         auto step = [&](int i, Pre& pr) {
             const bool live = i < n_iter;
-            if (live) stage_write(pr, qd(b3), meta_s4[b3]);
+            if (live) stage_write(pr, meta_s4[b3]);
+            wait_vmcnt<0>();      // this wave's part of tiles i and i+1 has landed
             __syncthreads();
             if (i >= 2) copy_out(dst(i & 1), h_q[0], r_q[0]);
-            if (i + 2 < n_iter) fetch(pr);
+            // tile i+2 replaces tile i-2, whose last readers finished before this barrier
+            if (i + 2 < n_iter) fetch(pr, (i + 2) & 3);
             const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
             if (!d_role) {
-                if (live) p_step(tail_c, qd(b3), meta_s4[b3], pbf(i & 1));
+                if (live) p_step(tail_c, qd(i & 3), meta_s4[b3], pbf(i & 1));
             } else {
-                // VALU-heavy half first: it overlaps the S MFMAs of the P-wave on this SIMD,
-                // whose exp2 phase then overlaps the dK MFMAs issued here
-                if (i >= 1) d_step_ds(qd(b3p), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), dp);
-                if (live) d_step_dp(qd(b3), dp);
+                d_step(i >= 1, live, qd((i - 1) & 3), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), qd(i & 3), dp);
             }
             shift();
             b3 = b3 == 2 ? 0 : b3 + 1;
@@ -328,9 +373,9 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // queue h_q/r_q: a tile enters at [4] when fetched; after k shifts it sits at
         // [4-k].  Tile i is fetched two steps ahead, so at step i (before that
         // step's shift) tile i is at [2], tile i-1 at [1], tile i-2 at [0].
-        fetch(preA);
+        fetch(preA, 0);
         shift();
-        if (n_iter > 1) fetch(preB);
+        if (n_iter > 1) fetch(preB, 1);
         shift();
         for (int i = 0; i <= n_iter; i += 2) {
             step(i, preA);
