@@ -265,8 +265,9 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // ---- D-wave.  For the previous tile (have_prev): dS = P (dP - delta) scale, dS^T to
     // LDS, dK_w^T += Q^T dS; for the current tile (live): dP = dO V_w^T.  All LDS operands
     // of both halves are requested first.
-    auto d_step = [&](bool have_prev, bool live, const uint16_t* qd_prev, const u32x4* meta, const uint16_t* pbuf,
+    auto d_step = [&](auto prev_c, auto live_c, const uint16_t* qd_prev, const u32x4* meta, const uint16_t* pbuf,
                       uint16_t* dst, const uint16_t* qd_cur, f32x16& dp) {
+        constexpr bool have_prev = decltype(prev_c)::value, live = decltype(live_c)::value;
         const char* qt = reinterpret_cast<const char*>(qd_prev);
         const char* dor = reinterpret_cast<const char*>(qd_cur) + TILE_ELEMS * 2;
         u32x4 pu[2];
@@ -330,7 +331,13 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
     };
 
-    auto run = [&](auto tail_c) {
+    // The loop exists once per role (no branch on the role inside it) and its first
+    // two steps and the draining step are peeled, so the steady-state step has no
+    // branch around code that updates the accumulators.
+    auto run = [&](auto tail_c, auto role_c) {
+        constexpr bool DROLE = decltype(role_c)::value;
+        using T = std::true_type;
+        using F = std::false_type;
         if (n_iter == 0) return;
         // tile i lives in qd(i & 3), its row metadata in meta_s4[i % 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
         auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
@@ -351,21 +358,21 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         f32x16 dp;
         int b3 = 0;   // i % 3
 
-        // Step i: stage tile i; P-waves do tile i; D-waves finish tile i-1 (dS, dK) and
-        // start tile i (dP); everyone copies dS^T(i-2) out.  Step n_iter only drains.
-        auto step = [&](int i, Pre& pr) {
-            const bool live = i < n_iter;
-            if (live) stage_write(pr, meta_s4[b3]);
+        // Step i: row metadata of tile i to LDS; P-waves do tile i; D-waves finish tile i-1
+        // (dS, dK) and start tile i (dP); everyone copies dS^T(i-2) out and requests tile i+2.
+        auto step = [&](auto prev_c, auto live_c, auto copy_c, int i, Pre& pr) {
+            constexpr bool LIVE = decltype(live_c)::value, COPY = decltype(copy_c)::value;
+            if (LIVE) stage_write(pr, meta_s4[b3]);
             wait_vmcnt<0>();      // this wave's part of tiles i and i+1 has landed
             __syncthreads();
-            if (i >= 2) copy_out(dst(i & 1), h_q[0], r_q[0]);
+            if (COPY) copy_out(dst(i & 1), h_q[0], r_q[0]);
             // tile i+2 replaces tile i-2, whose last readers finished before this barrier
             if (i + 2 < n_iter) fetch(pr, (i + 2) & 3);
             const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
-            if (!d_role) {
-                if (live) p_step(tail_c, qd(i & 3), meta_s4[b3], pbf(i & 1));
+            if (!DROLE) {
+                if (LIVE) p_step(tail_c, qd(i & 3), meta_s4[b3], pbf(i & 1));
             } else {
-                d_step(i >= 1, live, qd((i - 1) & 3), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), qd(i & 3), dp);
+                d_step(prev_c, live_c, qd((i - 1) & 3), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), qd(i & 3), dp);
             }
             shift();
             b3 = b3 == 2 ? 0 : b3 + 1;
@@ -373,19 +380,32 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // queue h_q/r_q: a tile enters at [4] when fetched; after k shifts it sits at
         // [4-k].  Tile i is fetched two steps ahead, so at step i (before that
         // step's shift) tile i is at [2], tile i-1 at [1], tile i-2 at [0].
+        // Tiles of even index travel through preA, of odd index through preB.
         fetch(preA, 0);
         shift();
         if (n_iter > 1) fetch(preB, 1);
         shift();
-        for (int i = 0; i <= n_iter; i += 2) {
-            step(i, preA);
-            if (i + 1 <= n_iter) step(i + 1, preB);
+        step(F{}, T{}, F{}, 0, preA);
+        if (n_iter == 1) {
+            step(T{}, F{}, F{}, 1, preB);
+        } else {
+            step(T{}, T{}, F{}, 1, preB);
+            for (int i = 2; i < n_iter; ++i) {
+                step(T{}, T{}, T{}, i, preA);
+                const Pre t = preA; preA = preB; preB = t;
+            }
+            step(T{}, F{}, T{}, n_iter, preA);
         }
         __syncthreads();
         copy_out(dst((n_iter - 1) & 1), h_q[0], r_q[0]);
     };
-    if (tail_block) run(std::true_type{});
-    else run(std::false_type{});
+    if (d_role) {
+        if (tail_block) run(std::true_type{}, std::true_type{});
+        else run(std::false_type{}, std::true_type{});
+    } else {
+        if (tail_block) run(std::true_type{}, std::false_type{});
+        else run(std::false_type{}, std::false_type{});
+    }
 
     // ---- epilogue: rows of acc = head-dim, cols = this wave's tokens; P-waves hold dV^T, D-waves dK^T
     if (p.dkv_mode == 2) {
