@@ -363,9 +363,14 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         auto step = [&](auto prev_c, auto live_c, auto copy_c, int i, Pre& pr) {
             constexpr bool LIVE = decltype(live_c)::value, COPY = decltype(copy_c)::value;
             if (LIVE) stage_write(pr, meta_s4[b3]);
-            wait_vmcnt<0>();      // this wave's part of tiles i and i+1 has landed
-            __syncthreads();
-            if (COPY) copy_out(dst(i & 1), h_q[0], r_q[0]);
+            // This wave's part of tile i (requested two steps ago) must have landed.  Since
+            // then it has issued 6 more vector-memory operations when the previous step
+            // requested a tile (metadata load, dS^T store; 2 tile loads, metadata load, store),
+            // 4 of them loads, and loads complete in order: at most 4 outstanding is enough,
+            // and leaves tile i+1 in flight.
+            if (i + 1 < n_iter) wait_vmcnt<4>();
+            else wait_vmcnt<0>();
+            lds_barrier();
             // tile i+2 replaces tile i-2, whose last readers finished before this barrier
             if (i + 2 < n_iter) fetch(pr, (i + 2) & 3);
             const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
@@ -374,6 +379,9 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             } else {
                 d_step(prev_c, live_c, qd((i - 1) & 3), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), qd(i & 3), dp);
             }
+            // dS^T(i-2) to HBM last: its LDS read queues behind this step's operand reads
+            // instead of delaying them, and only has to finish before the next barrier
+            if (COPY) copy_out(dst(i & 1), h_q[0], r_q[0]);
             shift();
             b3 = b3 == 2 ? 0 : b3 + 1;
         };
@@ -390,10 +398,14 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             step(T{}, F{}, F{}, 1, preB);
         } else {
             step(T{}, T{}, F{}, 1, preB);
-            for (int i = 2; i < n_iter; ++i) {
+            // two steps per trip: the metadata registers alternate without being moved
+            // (a move would have to wait for the load that is still filling them)
+            int i = 2;
+            for (; i + 1 < n_iter; i += 2) {
                 step(T{}, T{}, T{}, i, preA);
-                const Pre t = preA; preA = preB; preB = t;
+                step(T{}, T{}, T{}, i + 1, preB);
             }
+            if (i < n_iter) step(T{}, T{}, T{}, i, preA);
             step(T{}, F{}, T{}, n_iter, preA);
         }
         __syncthreads();

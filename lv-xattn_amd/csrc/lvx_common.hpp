@@ -116,6 +116,11 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Work-group barrier that orders LDS traffic only: this wave's LDS accesses are
+// complete before it and (being a compiler memory barrier too) none moves across
+// it, but vector-memory operations in flight - loads straight to LDS that are
+// waited for separately, stores - are not waited for, as __syncthreads() would.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // max of three (one instruction; fmaxf chains cost an extra canonicalising
 // v_max per MFMA result)
