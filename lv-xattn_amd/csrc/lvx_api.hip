@@ -231,8 +231,10 @@ size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
     if (!s || row_count <= 0) return 0;
     const size_t tokens = ((size_t)s->Lkv + 127) / 128 * 128;
     const size_t rows = ((size_t)row_count + 31) / 32 * 32;
-    // dS^T tiles, then fp32 dK/dV scratch for the split-steps mode with bf16 outputs
-    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s);
+    // dS^T tiles, then fp32 dK/dV scratch for the split-steps mode with bf16 outputs, then the
+    // row metadata records (2 floats per row and head)
+    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s) +
+           (size_t)s->B * s->Hq * rows * 2 * sizeof(float);
 }
 
 int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
@@ -263,7 +265,6 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
     p.dout = static_cast<const uint16_t*>(dout->ptr);
-    p.lse = lse; p.delta = delta;
     p.dk = dk->ptr; p.dv = dv->ptr;
     p.qs = st3(q); p.ks = st3(k); p.vs = st3(v); p.dos = st3(dout); p.dks = st3(dk); p.dvs = st3(dv);
     p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
@@ -276,6 +277,15 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.ds_ws = static_cast<uint16_t*>(workspace);
     p.ws_ld = rows * 128;          // one token block: (rows / 32) tiles of 128 x 32
     p.ws_bh = tokens * rows;
+
+    {
+        float* meta = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                               (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s));
+        MetaParams mp{lse, delta, meta, s->B, s->Hq, s->Lq, row_begin, row_begin + row_count, (int)(rows / 32), s->scale};
+        hipError_t em = launch_bwd_meta(mp, st);
+        if (em != hipSuccess) return static_cast<int>(em);
+        p.meta = meta;
+    }
 
     const int blocks = s->B * s->Hkv * p.n_kv_blocks;
     const int steps = p.G * (int)(rows / 32);

@@ -70,9 +70,9 @@ constexpr float LOG2E = 1.4426950408889634f;
 template <bool MASKED>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
-    // per-row metadata of a staged tile, triple-buffered: 8 x 16 bytes each of
-    // LSE*log2e, delta, kv_start, kv_end
-    __shared__ u32x4 meta_s4[3][BM];
+    // per-row metadata of a staged tile, one per tile buffer: 8 x 16 bytes each of
+    // LSE*log2e, delta*scale, kv_start, kv_end
+    __shared__ __attribute__((aligned(256))) u32x4 meta_s4[NQD][BM];
 
     const int wid = xcd_remap(blockIdx.x, p.total_wg);
     if (wid >= p.total_wg) return;
@@ -122,17 +122,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const uint32_t ld_c = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | (wave & 3))) * 16u;
     const uint32_t qrow_b = (uint32_t)p.qs.s * 2u, dorow_b = (uint32_t)p.dos.s * 2u;   // bytes per text row
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-    const int meta_kind = (tid >> 5) & 3;    // 0 LSE, 1 delta, 2 kv_start, 3 kv_end (threads 0..127)
-    const uint32_t* m_base = reinterpret_cast<const uint32_t*>(p.lse);
-    int64_t m_hs = p.Lq;
-    if (meta_kind == 1) m_base = reinterpret_cast<const uint32_t*>(p.delta);
-    if (MASKED && meta_kind >= 2) {
-        m_base = reinterpret_cast<const uint32_t*>(meta_kind == 2 ? p.kv_start : p.kv_end) + (int64_t)b * p.Lq;
-        m_hs = 0;
-    } else {
-        m_base += (int64_t)b * p.Hq * p.Lq;
-    }
-
+    const uint32_t meta0 = (uint32_t)(uintptr_t)&meta_s4[0][0];
     // per-lane offsets: transposing operand reads (rows in accumulator order),
     // P hand-over slot, dS^T copy-out (512 chunks of 16 bytes, one per thread)
     // rows: 16 bytes at row * 256 + ((2 kk + g) ^ f(row)) * 16
@@ -157,27 +147,28 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     int cur_gi = it_lo / n_qtiles, cur_qt = it_lo % n_qtiles;
 
-    // Every load is unconditional: rows past the window are clamped to its last
-    // row (their LSE is forced to +inf, so P = 0 and nothing they carry reaches a
-    // result), and the fetch after the last tile re-reads some tile.
-    // The Q / dO tile goes straight to its LDS buffer; the row metadata travels
-    // through one of two alternating register pairs and is stored two steps later.
-    struct Pre {
-        uint32_t m;
-        bool ok;
-    };
-    Pre preA{}, preB{};
-    auto prefetch = [&](Pre& pr, int buf) {
+    // Every load is unconditional and goes straight to LDS: rows past the window are
+    // clamped to its last row (their LSE record is +inf, so P = 0 and nothing they
+    // carry reaches a result).  Wave 0 also fetches the tile's metadata record
+    // (32 x LSE*log2e, 32 x delta*scale; 256 bytes) and, with a mask, the rows'
+    // key intervals, ahead of its tile loads so that "tile landed" implies both.
+    auto prefetch = [&](int buf) {
         const int h = hk * p.G + cur_gi;
         const int r0 = p.row_begin + cur_qt * BM;
+        if (wave == 0) {
+            const uint32_t mslot = meta0 + (uint32_t)buf * (BM * 16);
+            const float* rec = p.meta + (((int64_t)b * p.Hq + h) * n_qtiles + cur_qt) * 64;
+            dma4(reinterpret_cast<const char*>(rec), (uint32_t)lane * 4u, mslot);
+            if (MASKED) {
+                const int32_t* iv = (lane < 32 ? p.kv_start : p.kv_end) + (int64_t)b * p.Lq + min(r0 + l32, p.row_end - 1);
+                dma4_addr(reinterpret_cast<const char*>(iv), mslot + 256);
+            }
+        }
         const uint32_t row = (uint32_t)min(r0 + ld_r, p.row_end - 1);
         const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)wave * 1024u;
         dma16(reinterpret_cast<const char*>(p.q + b * p.qs.b + h * p.qs.h), row * qrow_b + ld_c, slot);
         dma16(reinterpret_cast<const char*>(p.dout + b * p.dos.b + h * p.dos.h), row * dorow_b + ld_c,
               slot + TILE_ELEMS * 2);
-        const int mrow = r0 + (tid & 31);
-        pr.ok = mrow < p.row_end;
-        pr.m = m_base[h * m_hs + min(mrow, p.row_end - 1)];
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
         if (++cur_qt == n_qtiles) {
@@ -185,14 +176,6 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             if (++cur_gi == p.G) cur_gi = 0;
         }
     };
-    auto stage_write = [&](const Pre& pr, u32x4* meta) {
-        const float l = __uint_as_float(pr.m);
-        // exp2(x - inf) = 0: rows that saw no key (or do not exist) get P = 0
-        const float lt = (!pr.ok || l == -INFINITY) ? INFINITY : l * LOG2E;
-        const uint32_t m = meta_kind == 0 ? __float_as_uint(lt) : (pr.ok ? pr.m : 0u);
-        reinterpret_cast<uint32_t*>(meta)[tid & 127] = m;   // the four quarters write the same words
-    };
-
     // the finished dS^T tile goes to HBM as one contiguous 8 KB block
     auto copy_out = [&](const uint16_t* dst, int h, int r0) {
         uint16_t* gp = ws_lane + ((int64_t)b * p.Hq + h) * p.ws_bh + (int64_t)((r0 - p.row_begin) / BM) * (BN * BM);
@@ -296,8 +279,9 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                     // registers 8j + 2e, 8j + 2e + 1 are rows 16j + 8(e/2) + 4g + 2(e%2) + {0, 1}
                     const float d0 = (e < 2) ? da4[2 * (e & 1)] : db4[2 * (e & 1)];
                     const float d1 = (e < 2) ? da4[2 * (e & 1) + 1] : db4[2 * (e & 1) + 1];
-                    const float p0 = bf16_lo(pu[j][e]) * p.scale, p1 = bf16_hi(pu[j][e]) * p.scale;
-                    dsu[j][e] = pack_bf16(p0 * (dp[8 * j + 2 * e] - d0), p1 * (dp[8 * j + 2 * e + 1] - d1));
+                    // scale * P * (dP - delta), with delta * scale from the record
+                    dsu[j][e] = pack_bf16(bf16_lo(pu[j][e]) * fmaf(dp[8 * j + 2 * e], p.scale, -d0),
+                                          bf16_hi(pu[j][e]) * fmaf(dp[8 * j + 2 * e + 1], p.scale, -d1));
                 }
             }
             uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
@@ -339,16 +323,16 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         using T = std::true_type;
         using F = std::false_type;
         if (n_iter == 0) return;
-        // tile i lives in qd(i & 3), its row metadata in meta_s4[i % 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
+        // tile i lives in qd(i & 3), its row metadata in meta_s4[i & 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
         auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
         auto dst = [&](int k) { return smem + OFF_DST + k * DST_ELEMS; };
         auto pbf = [&](int k) { return smem + OFF_PB + k * PB_ELEMS; };
         // (h, r0) of the tiles: being fetched (+2, +1), current (0), previous (-1, -2)
         int h_q[5] = {0, 0, 0, 0, 0}, r_q[5] = {0, 0, 0, 0, 0};
-        auto fetch = [&](Pre& pr, int buf) {   // start the loads of the next tile of the walk
+        auto fetch = [&](int buf) {   // start the loads of the next tile of the walk
             h_q[4] = hk * p.G + cur_gi;
             r_q[4] = p.row_begin + cur_qt * BM;
-            prefetch(pr, buf);
+            prefetch(buf);
             advance();
         };
         auto shift = [&]() {
@@ -356,57 +340,45 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             for (int k = 0; k < 4; ++k) { h_q[k] = h_q[k + 1]; r_q[k] = r_q[k + 1]; }
         };
         f32x16 dp;
-        int b3 = 0;   // i % 3
 
-        // Step i: row metadata of tile i to LDS; P-waves do tile i; D-waves finish tile i-1
-        // (dS, dK) and start tile i (dP); everyone copies dS^T(i-2) out and requests tile i+2.
-        auto step = [&](auto prev_c, auto live_c, auto copy_c, int i, Pre& pr) {
+        // Step i: P-waves do tile i; D-waves finish tile i-1 (dS, dK) and start tile i
+        // (dP); everyone requests tile i+2 and copies dS^T(i-2) out.
+        auto step = [&](auto prev_c, auto live_c, auto copy_c, int i) {
             constexpr bool LIVE = decltype(live_c)::value, COPY = decltype(copy_c)::value;
-            if (LIVE) stage_write(pr, meta_s4[b3]);
-            // This wave's part of tile i (requested two steps ago) must have landed.  Since
-            // then it has issued 6 more vector-memory operations when the previous step
-            // requested a tile (metadata load, dS^T store; 2 tile loads, metadata load, store),
-            // 4 of them loads, and loads complete in order: at most 4 outstanding is enough,
-            // and leaves tile i+1 in flight.
-            if (i + 1 < n_iter) wait_vmcnt<4>();
+            // This wave's part of tile i (requested two steps ago) must have landed.  When
+            // the previous step requested a tile, the wave has issued since: a dS^T store,
+            // [wave 0: metadata loads,] 2 tile loads, a store.  Loads complete in order, so
+            // "at most 2 operations outstanding" covers tile i and leaves tile i+1 in flight.
+            if (i + 1 < n_iter) wait_vmcnt<2>();
             else wait_vmcnt<0>();
             lds_barrier();
             // tile i+2 replaces tile i-2, whose last readers finished before this barrier
-            if (i + 2 < n_iter) fetch(pr, (i + 2) & 3);
-            const int b3p = b3 == 0 ? 2 : b3 - 1;   // (i - 1) % 3
+            if (i + 2 < n_iter) fetch((i + 2) & 3);
             if (!DROLE) {
-                if (LIVE) p_step(tail_c, qd(i & 3), meta_s4[b3], pbf(i & 1));
+                if (LIVE) p_step(tail_c, qd(i & 3), meta_s4[i & 3], pbf(i & 1));
             } else {
-                d_step(prev_c, live_c, qd((i - 1) & 3), meta_s4[b3p], pbf((i - 1) & 1), dst((i - 1) & 1), qd(i & 3), dp);
+                d_step(prev_c, live_c, qd((i - 1) & 3), meta_s4[(i - 1) & 3], pbf((i - 1) & 1), dst((i - 1) & 1),
+                       qd(i & 3), dp);
             }
             // dS^T(i-2) to HBM last: its LDS read queues behind this step's operand reads
             // instead of delaying them, and only has to finish before the next barrier
             if (COPY) copy_out(dst(i & 1), h_q[0], r_q[0]);
             shift();
-            b3 = b3 == 2 ? 0 : b3 + 1;
         };
         // queue h_q/r_q: a tile enters at [4] when fetched; after k shifts it sits at
         // [4-k].  Tile i is fetched two steps ahead, so at step i (before that
         // step's shift) tile i is at [2], tile i-1 at [1], tile i-2 at [0].
-        // Tiles of even index travel through preA, of odd index through preB.
-        fetch(preA, 0);
+        fetch(0);
         shift();
-        if (n_iter > 1) fetch(preB, 1);
+        if (n_iter > 1) fetch(1);
         shift();
-        step(F{}, T{}, F{}, 0, preA);
+        step(F{}, T{}, F{}, 0);
         if (n_iter == 1) {
-            step(T{}, F{}, F{}, 1, preB);
+            step(T{}, F{}, F{}, 1);
         } else {
-            step(T{}, T{}, F{}, 1, preB);
-            // two steps per trip: the metadata registers alternate without being moved
-            // (a move would have to wait for the load that is still filling them)
-            int i = 2;
-            for (; i + 1 < n_iter; i += 2) {
-                step(T{}, T{}, T{}, i, preA);
-                step(T{}, T{}, T{}, i + 1, preB);
-            }
-            if (i < n_iter) step(T{}, T{}, T{}, i, preA);
-            step(T{}, F{}, T{}, n_iter, preA);
+            step(T{}, T{}, F{}, 1);
+            for (int i = 2; i < n_iter; ++i) step(T{}, T{}, T{}, i);
+            step(T{}, F{}, T{}, n_iter);
         }
         __syncthreads();
         copy_out(dst((n_iter - 1) & 1), h_q[0], r_q[0]);

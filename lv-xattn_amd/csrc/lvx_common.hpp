@@ -111,6 +111,14 @@ __device__ __forceinline__ void dma16(const char* sbase, uint32_t voff, uint32_t
 __device__ __forceinline__ void dma16_addr(const char* addr, uint32_t lds_byte) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte), "v"(addr) : "memory", "m0");
 }
+// the same with 4 bytes per lane: lane i lands at lds_byte + 4 i
+__device__ __forceinline__ void dma4(const char* sbase, uint32_t voff, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_byte), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma4_addr(const char* addr, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_byte), "v"(addr) : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

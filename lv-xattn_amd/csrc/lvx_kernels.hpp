@@ -59,8 +59,7 @@ struct BwdParams {
     const uint16_t* k;
     const uint16_t* v;
     const uint16_t* dout;
-    const float* lse;
-    const float* delta;
+    const float* meta;         // per (b, h, 32-row tile): 32 x LSE*log2(e) (+inf for dead rows), 32 x delta*scale
     uint16_t* ds_ws;           // dS^T workspace [B*Hq][token blocks][row tiles][128 tokens][32 rows]
     int64_t ws_ld;             // elements per token block (row tiles * 4096)
     int64_t ws_bh;             // elements per (b, h) slab
@@ -77,6 +76,16 @@ struct BwdParams {
     int split_steps;           // steps (32-row tiles x heads of the group) per split
     int dkv_mode;              // 0: store bf16, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1)
     float scale, scale_log2e;
+};
+
+// Row metadata of the backward in the form its kernel consumes, one 256-byte
+// record per (b, h, 32-row tile of the window).
+struct MetaParams {
+    const float* lse;
+    const float* delta;
+    float* out;
+    int B, Hq, Lq, row_begin, row_end, n_tiles;
+    float scale;
 };
 
 struct FillParams {
@@ -126,6 +135,7 @@ hipError_t launch_merge(const MergeParams& p, hipStream_t st);
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st);
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);
 hipError_t launch_cast(const CastParams& p, hipStream_t st);
+hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st);
 hipError_t launch_zero(const FillParams& p, hipStream_t st);
 // a_mcontig: A is stored [K][M] (m contiguous); b_ncontig: B is stored [K][N].
 hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st);

@@ -110,6 +110,25 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
     if (ok && chunk == 0) p.delta[(int64_t)bh * p.Lq + row] = s;
 }
 
+// LSE and delta of the window, re-expressed once for the backward kernel: the
+// exponent offset LSE * log2(e), +inf for rows that saw no key or lie past the
+// window (so that P = exp2(x - inf) = 0 there), and delta * scale (0 past the
+// window), grouped per 32-row tile so that one 256-byte load fetches a tile's lot.
+__global__ __launch_bounds__(256) void bwd_meta_kernel(const MetaParams p) {
+    const int rows_pad = p.n_tiles * 32;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.B * p.Hq * rows_pad) return;
+    const int r = (int)(idx % rows_pad);
+    const int64_t bh = idx / rows_pad;
+    const int row = p.row_begin + r;
+    const bool ok = row < p.row_end;
+    const float l = ok ? p.lse[bh * p.Lq + row] : -INFINITY;
+    const float d = ok ? p.delta[bh * p.Lq + row] : 0.f;
+    float* o = p.out + (bh * p.n_tiles + (r >> 5)) * 64 + (r & 31);
+    o[0] = (l == -INFINITY) ? INFINITY : l * 1.4426950408889634f;
+    o[32] = d * p.scale;
+}
+
 __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
@@ -150,6 +169,13 @@ hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
     hipLaunchKernelGGL(preprocess_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st) {
+    const int64_t n = (int64_t)p.B * p.Hq * p.n_tiles * 32;
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(bwd_meta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
