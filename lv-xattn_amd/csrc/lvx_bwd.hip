@@ -27,7 +27,7 @@
 //
 // All MFMA are 32x32x16 bf16.  A operands come from LDS.  The Q and dO tiles
 // ([32 rows][128] bf16, 8 KiB each) go from global memory straight into LDS
-// with global_load_lds_dwordx4, two steps ahead, into a ring of four buffers;
+// with global_load_lds_dwordx4, two steps ahead, into a ring of five buffers;
 // the load writes 64 lanes x 16 bytes contiguously, so rows are not padded:
 // the 16-byte chunk c of row r is kept at position c ^ f(r),
 // f(r) = ((r & 3) << 2) | ((r >> 2) & 3), which makes both access patterns
@@ -54,10 +54,10 @@ constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row]
 // LDS map (uint16 units): four (Q | dO) tile pairs, unpadded; two dS^T tiles; two P hand-over buffers
 constexpr int TILE_ELEMS = BM * D;             // one Q or dO tile (8 KiB)
 constexpr int QD_ELEMS = 2 * TILE_ELEMS;
-constexpr int NQD = 4;
+constexpr int NQD = 5;
 constexpr int DST_ELEMS = BN * DSS;
 constexpr int PB_ELEMS = 4 * 2 * 64 * 8;       // P hand-over: [slice][half][lane][16 bytes] as uint16
-constexpr int OFF_QD = 0;                      // x4
+constexpr int OFF_QD = 0;                      // x NQD
 constexpr int OFF_DST = OFF_QD + NQD * QD_ELEMS; // x2
 constexpr int OFF_PB = OFF_DST + 2 * DST_ELEMS;  // x2
 constexpr int LOOP_ELEMS = OFF_PB + 2 * PB_ELEMS;
@@ -145,7 +145,21 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // workspace tile (b, h, token block, row tile): [128 tokens][32 rows], 8 KB, contiguous
     uint16_t* ws_lane = p.ds_ws + (int64_t)kblk * p.ws_ld + cp_token * BM + cp_part * 8;
 
+    // The walk over (head of the group, 32-row tile): per-head base addresses are
+    // re-derived only when the head changes, everything else advances by constants.
     int cur_gi = it_lo / n_qtiles, cur_qt = it_lo % n_qtiles;
+    const char* q_head = nullptr;      // Q, dO of (b, head)
+    const char* do_head = nullptr;
+    const float* meta_head = nullptr;  // metadata records of (b, head)
+    int64_t ws_head = 0;               // dS^T workspace offset of (b, head), elements
+    auto enter_head = [&]() {
+        const int h = hk * p.G + cur_gi;
+        q_head = reinterpret_cast<const char*>(p.q + b * p.qs.b + h * p.qs.h);
+        do_head = reinterpret_cast<const char*>(p.dout + b * p.dos.b + h * p.dos.h);
+        meta_head = p.meta + ((int64_t)b * p.Hq + h) * n_qtiles * 64;
+        ws_head = ((int64_t)b * p.Hq + h) * p.ws_bh;
+    };
+    enter_head();
 
     // Every load is unconditional and goes straight to LDS: rows past the window are
     // clamped to its last row (their LSE record is +inf, so P = 0 and nothing they
@@ -153,12 +167,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // (32 x LSE*log2e, 32 x delta*scale; 256 bytes) and, with a mask, the rows'
     // key intervals, ahead of its tile loads so that "tile landed" implies both.
     auto prefetch = [&](int buf) {
-        const int h = hk * p.G + cur_gi;
         const int r0 = p.row_begin + cur_qt * BM;
         if (wave == 0) {
             const uint32_t mslot = meta0 + (uint32_t)buf * (BM * 16);
-            const float* rec = p.meta + (((int64_t)b * p.Hq + h) * n_qtiles + cur_qt) * 64;
-            dma4(reinterpret_cast<const char*>(rec), (uint32_t)lane * 4u, mslot);
+            dma4(reinterpret_cast<const char*>(meta_head + cur_qt * 64), (uint32_t)lane * 4u, mslot);
             if (MASKED) {
                 const int32_t* iv = (lane < 32 ? p.kv_start : p.kv_end) + (int64_t)b * p.Lq + min(r0 + l32, p.row_end - 1);
                 dma4_addr(reinterpret_cast<const char*>(iv), mslot + 256);
@@ -166,99 +178,128 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
         const uint32_t row = (uint32_t)min(r0 + ld_r, p.row_end - 1);
         const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)wave * 1024u;
-        dma16(reinterpret_cast<const char*>(p.q + b * p.qs.b + h * p.qs.h), row * qrow_b + ld_c, slot);
-        dma16(reinterpret_cast<const char*>(p.dout + b * p.dos.b + h * p.dos.h), row * dorow_b + ld_c,
-              slot + TILE_ELEMS * 2);
+        dma16(q_head, row * qrow_b + ld_c, slot);
+        dma16(do_head, row * dorow_b + ld_c, slot + TILE_ELEMS * 2);
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
         if (++cur_qt == n_qtiles) {
             cur_qt = 0;
             if (++cur_gi == p.G) cur_gi = 0;
+            enter_head();
         }
-    };
-    // the finished dS^T tile goes to HBM as one contiguous 8 KB block
-    auto copy_out = [&](const uint16_t* dst, int h, int r0) {
-        uint16_t* gp = ws_lane + ((int64_t)b * p.Hq + h) * p.ws_bh + (int64_t)((r0 - p.row_begin) / BM) * (BN * BM);
-        *reinterpret_cast<u32x4*>(gp) = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
     };
 
-    // ---- P-wave: S = Q K_w^T, P = exp2(S*c - LSE*log2e) (masked), hand P over, dV_w^T += dO^T P
-    auto p_step = [&](auto tail_c, const uint16_t* qd, const u32x4* meta, uint16_t* pbuf) {
+    // the finished dS^T tile goes to HBM as one contiguous 8 KB block
+    auto copy_out = [&](const uint16_t* dst, int64_t ws_off) {
+        *reinterpret_cast<u32x4*>(ws_lane + ws_off) = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
+    };
+
+    // The work on a tile is spread over three steps so that, inside every wave, the
+    // MFMAs of one tile and the VALU work of an earlier tile are independent and
+    // overlap (on top of the overlap between the two waves of a SIMD):
+    //   step i, P-wave: S(i) = Q K_w^T                     || P(i-1) = exp2(S(i-1)*c - LSE*log2e), masked
+    //                   then hand P(i-1) over, dV_w^T += dO(i-1)^T P(i-1)
+    //   step i, D-wave: dP(i-1) = dO V_w^T                 || dS(i-2) = P(i-2) (dP(i-2)*scale - delta*scale)
+    //                   then dS^T(i-2) to LDS, dK_w^T += Q(i-2)^T dS(i-2)
+    //   step i, all   : request tile i+2, copy dS^T(i-3) out
+    // Flags say which halves exist at the edges of the walk; they are compile-time
+    // constants in the steady-state loop.
+    auto p_step = [&](auto tail_c, bool s_live, bool pv_live, const uint16_t* tile_cur, const uint16_t* tile_prev,
+                      const u32x4* meta, uint16_t* pbuf, f32x16& s_carry) __attribute__((always_inline)) {
         constexpr bool TAIL = decltype(tail_c)::value;
-        const char* qt = reinterpret_cast<const char*>(qd);
-        const char* dot = qt + TILE_ELEMS * 2;
+        const char* qt = reinterpret_cast<const char*>(tile_cur);
+        const char* dot = reinterpret_cast<const char*>(tile_prev) + TILE_ELEMS * 2;
         bf16x8 qa[8];
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk)
-            qa[kk] = *reinterpret_cast<const bf16x8*>(qt + row_rd + ((uint32_t)(kk * 32) ^ row_h));
-        __builtin_amdgcn_sched_barrier(0);
-        f32x16 s;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) s = mfma32(qa[kk], breg[kk], s);
-        __builtin_amdgcn_sched_barrier(0);
-        // dO^T operands: requested now, they land during the exp2 phase
         u32x2 da[4][2][2];
+        if (s_live) {
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                da[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][0] + j * 4096));
-                da[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][1] + j * 4096));
-            }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int vg = 0; vg < 4; ++vg) {
-            const f32x4 l4 = __builtin_bit_cast(f32x4, meta[2 * vg + g]);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) s[4 * vg + r] = __builtin_amdgcn_exp2f(fmaf(s[4 * vg + r], c, -l4[r]));
+            for (int kk = 0; kk < 8; ++kk)
+                qa[kk] = *reinterpret_cast<const bf16x8*>(qt + row_rd + ((uint32_t)(kk * 32) ^ row_h));
         }
-        if (MASKED) {
+        __builtin_amdgcn_sched_barrier(0);
+        f32x16 s_new;
+        if (s_live) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_new[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) s_new = mfma32(qa[kk], breg[kk], s_new);
+        }
+        if (pv_live) {
+            // dO^T operands: requested once the S operands are consumed; they land while
+            // the exp2 phase runs in the shadow of the S MFMAs
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    da[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][0] + j * 4096));
+                    da[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][1] + j * 4096));
+                }
+            f32x16 s = s_carry;
 #pragma unroll
             for (int vg = 0; vg < 4; ++vg) {
-                const u32x4 sp = meta[16 + 2 * vg + g];
-                const u32x4 ep = meta[24 + 2 * vg + g];
+                const f32x4 l4 = __builtin_bit_cast(f32x4, meta[2 * vg + g]);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
-                    s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
+                for (int r = 0; r < 4; ++r) s[4 * vg + r] = __builtin_amdgcn_exp2f(fmaf(s[4 * vg + r], c, -l4[r]));
+            }
+            if (MASKED) {
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const u32x4 sp = meta[16 + 2 * vg + g];
+                    const u32x4 ep = meta[24 + 2 * vg + g];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
+                        s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
+                    }
                 }
-            }
-        } else if (TAIL) {
+            } else if (TAIL) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s[v] = kv_valid ? s[v] : 0.f;
+                for (int v = 0; v < 16; ++v) s[v] = kv_valid ? s[v] : 0.f;
+            }
+            u32x4 pu[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) pu[j][e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
+            *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
+            *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const u32x4 a = {da[dt][j][0][0], da[dt][j][0][1], da[dt][j][1][0], da[dt][j][1][1]};
+                    acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(pu[j]), acc[dt]);
+                }
         }
-        u32x4 pu[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) pu[j][e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
-        *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
-        *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const u32x4 a = {da[dt][j][0][0], da[dt][j][0][1], da[dt][j][1][0], da[dt][j][1][1]};
-                acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(pu[j]), acc[dt]);
-            }
+        if (s_live) s_carry = s_new;
     };
 
-    // ---- D-wave.  For the previous tile (have_prev): dS = P (dP - delta) scale, dS^T to
-    // LDS, dK_w^T += Q^T dS; for the current tile (live): dP = dO V_w^T.  All LDS operands
-    // of both halves are requested first.
-    auto d_step = [&](auto prev_c, auto live_c, const uint16_t* qd_prev, const u32x4* meta, const uint16_t* pbuf,
-                      uint16_t* dst, const uint16_t* qd_cur, f32x16& dp) {
-        constexpr bool have_prev = decltype(prev_c)::value, live = decltype(live_c)::value;
-        const char* qt = reinterpret_cast<const char*>(qd_prev);
-        const char* dor = reinterpret_cast<const char*>(qd_cur) + TILE_ELEMS * 2;
+    auto d_step = [&](bool pv_live, bool ds_live, const uint16_t* tile_p1, const uint16_t* tile_p2, const u32x4* meta,
+                      const uint16_t* pbuf, uint16_t* dst, f32x16& dp_carry) __attribute__((always_inline)) {
+        const char* dor = reinterpret_cast<const char*>(tile_p1) + TILE_ELEMS * 2;   // dO rows of tile i-1
+        const char* qt = reinterpret_cast<const char*>(tile_p2);                     // Q of tile i-2
         u32x4 pu[2];
         u32x2 qa[4][2][2];
         bf16x8 da[8];
-        if (have_prev) {
+        if (pv_live) {
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk)
+                da[kk] = *reinterpret_cast<const bf16x8*>(dor + row_rd + ((uint32_t)(kk * 32) ^ row_h));
+        }
+        if (ds_live) {
             pu[0] = *reinterpret_cast<const u32x4*>(pbuf + pb_off);
             pu[1] = *reinterpret_cast<const u32x4*>(pbuf + pb_off + 64 * 8);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        f32x16 dp_new;
+        if (pv_live) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dp_new[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) dp_new = mfma32(da[kk], breg[kk], dp_new);
+        }
+        if (ds_live) {
+            // Q^T operands: requested once the dO operands are consumed
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -266,10 +307,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                     qa[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(qt + t_rd[dt][0] + j * 4096));
                     qa[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(qt + t_rd[dt][1] + j * 4096));
                 }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        u32x4 dsu[2];
-        if (have_prev) {
+            u32x4 dsu[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const f32x4 da4 = __builtin_bit_cast(f32x4, meta[8 + 4 * j + g]);       // rows 16j + 4g + 0..3
@@ -280,8 +318,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                     const float d0 = (e < 2) ? da4[2 * (e & 1)] : db4[2 * (e & 1)];
                     const float d1 = (e < 2) ? da4[2 * (e & 1) + 1] : db4[2 * (e & 1) + 1];
                     // scale * P * (dP - delta), with delta * scale from the record
-                    dsu[j][e] = pack_bf16(bf16_lo(pu[j][e]) * fmaf(dp[8 * j + 2 * e], p.scale, -d0),
-                                          bf16_hi(pu[j][e]) * fmaf(dp[8 * j + 2 * e + 1], p.scale, -d1));
+                    dsu[j][e] = pack_bf16(bf16_lo(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e], p.scale, -d0),
+                                          bf16_hi(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e + 1], p.scale, -d1));
                 }
             }
             uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
@@ -290,15 +328,6 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 const u32x2 w = {dsu[vg >> 1][2 * (vg & 1)], dsu[vg >> 1][2 * (vg & 1) + 1]};
                 *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
             }
-        }
-        // dO rows of the current tile: in flight during the dK MFMAs
-        if (live) {
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk)
-                da[kk] = *reinterpret_cast<const bf16x8*>(dor + row_rd + ((uint32_t)(kk * 32) ^ row_h));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (have_prev) {
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -307,44 +336,36 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                     acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(dsu[j]), acc[dt]);
                 }
         }
-        if (live) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) dp[v] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) dp = mfma32(da[kk], breg[kk], dp);
-        }
+        if (pv_live) dp_carry = dp_new;
     };
 
-    // The loop exists once per role (no branch on the role inside it) and its first
-    // two steps and the draining step are peeled, so the steady-state step has no
-    // branch around code that updates the accumulators.
+    // The loop exists once per role (no branch on the role inside it).
     auto run = [&](auto tail_c, auto role_c) {
         constexpr bool DROLE = decltype(role_c)::value;
-        using T = std::true_type;
-        using F = std::false_type;
         if (n_iter == 0) return;
-        // tile i lives in qd(i & 3), its row metadata in meta_s4[i & 3]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
+        // tile i lives in qd(i % 5) with its row metadata in meta_s4[i % 5]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
         auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
         auto dst = [&](int k) { return smem + OFF_DST + k * DST_ELEMS; };
         auto pbf = [&](int k) { return smem + OFF_PB + k * PB_ELEMS; };
-        // (h, r0) of the tiles: being fetched (+2, +1), current (0), previous (-1, -2)
-        int h_q[5] = {0, 0, 0, 0, 0}, r_q[5] = {0, 0, 0, 0, 0};
+        auto m5 = [](int x) { return x >= NQD ? x - NQD : x; };
+        // dS^T workspace offsets of the tiles in flight: a tile enters at [5] when requested
+        // (two steps ahead); at step i (before that step's shift) tile i is at [3], tile i-3 at [0]
+        int64_t w_q[6] = {0, 0, 0, 0, 0, 0};
         auto fetch = [&](int buf) {   // start the loads of the next tile of the walk
-            h_q[4] = hk * p.G + cur_gi;
-            r_q[4] = p.row_begin + cur_qt * BM;
+            w_q[5] = ws_head + (int64_t)cur_qt * (BN * BM);
             prefetch(buf);
             advance();
         };
         auto shift = [&]() {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) { h_q[k] = h_q[k + 1]; r_q[k] = r_q[k + 1]; }
+            for (int k = 0; k < 5; ++k) w_q[k] = w_q[k + 1];
         };
-        f32x16 dp;
+        f32x16 carry;     // P-wave: raw S of the previous tile; D-wave: dP of the previous tile
+#pragma unroll
+        for (int v = 0; v < 16; ++v) carry[v] = 0.f;
+        int rc = 0;       // i % 5
 
-        // Step i: P-waves do tile i; D-waves finish tile i-1 (dS, dK) and start tile i
-        // (dP); everyone requests tile i+2 and copies dS^T(i-2) out.
-        auto step = [&](auto prev_c, auto live_c, auto copy_c, int i) {
-            constexpr bool LIVE = decltype(live_c)::value, COPY = decltype(copy_c)::value;
+        auto step = [&](int i, bool s_live, bool pv_live, bool ds_live, bool copy) __attribute__((always_inline)) {
             // This wave's part of tile i (requested two steps ago) must have landed.  When
             // the previous step requested a tile, the wave has issued since: a dS^T store,
             // [wave 0: metadata loads,] 2 tile loads, a store.  Loads complete in order, so
@@ -352,36 +373,30 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             if (i + 1 < n_iter) wait_vmcnt<2>();
             else wait_vmcnt<0>();
             lds_barrier();
-            // tile i+2 replaces tile i-2, whose last readers finished before this barrier
-            if (i + 2 < n_iter) fetch((i + 2) & 3);
-            if (!DROLE) {
-                if (LIVE) p_step(tail_c, qd(i & 3), meta_s4[i & 3], pbf(i & 1));
-            } else {
-                d_step(prev_c, live_c, qd((i - 1) & 3), meta_s4[(i - 1) & 3], pbf((i - 1) & 1), dst((i - 1) & 1),
-                       qd(i & 3), dp);
-            }
-            // dS^T(i-2) to HBM last: its LDS read queues behind this step's operand reads
+            // tile i+2 replaces tile i-3, whose last readers finished before this barrier
+            if (i + 2 < n_iter) fetch(m5(rc + 2));
+            const int r1 = m5(rc + 4), r2 = m5(rc + 3);     // (i - 1) % 5, (i - 2) % 5
+            if (!DROLE)
+                p_step(tail_c, s_live, pv_live, qd(rc), qd(r1), meta_s4[r1], pbf((i + 1) & 1), carry);
+            else
+                d_step(pv_live, ds_live, qd(r1), qd(r2), meta_s4[r2], pbf(i & 1), dst(i & 1), carry);
+            // dS^T(i-3) to HBM last: its LDS read queues behind this step's operand reads
             // instead of delaying them, and only has to finish before the next barrier
-            if (COPY) copy_out(dst(i & 1), h_q[0], r_q[0]);
+            if (copy) copy_out(dst((i + 1) & 1), w_q[0]);
             shift();
+            rc = m5(rc + 1);
         };
-        // queue h_q/r_q: a tile enters at [4] when fetched; after k shifts it sits at
-        // [4-k].  Tile i is fetched two steps ahead, so at step i (before that
-        // step's shift) tile i is at [2], tile i-1 at [1], tile i-2 at [0].
         fetch(0);
         shift();
         if (n_iter > 1) fetch(1);
         shift();
-        step(F{}, T{}, F{}, 0);
-        if (n_iter == 1) {
-            step(T{}, F{}, F{}, 1);
-        } else {
-            step(T{}, T{}, F{}, 1);
-            for (int i = 2; i < n_iter; ++i) step(T{}, T{}, T{}, i);
-            step(T{}, F{}, T{}, n_iter);
-        }
+        const int last = n_iter + 1;
+        int i = 0;
+        for (; i < 3 && i <= last; ++i) step(i, i < n_iter, i >= 1 && i <= n_iter, i >= 2, false);
+        for (; i < n_iter; ++i) step(i, true, true, true, true);
+        for (; i <= last; ++i) step(i, false, i <= n_iter, true, true);
         __syncthreads();
-        copy_out(dst((n_iter - 1) & 1), h_q[0], r_q[0]);
+        copy_out(dst((n_iter - 1) & 1), w_q[0]);
     };
     if (d_role) {
         if (tail_block) run(std::true_type{}, std::true_type{});
