@@ -14,6 +14,7 @@ Everything runs on the current PyTorch stream; nothing here synchronises.
 """
 from __future__ import annotations
 
+import math
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -51,11 +52,25 @@ def _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args):
             "pass the compact interval form via mask=Mask(kv_len, kv_start, kv_end)")
 
 
+def auto_kv_splits(B: int, Hq: int, Hkv: int, rows: int, Lkv: int, target_wgs: int = 512) -> int:
+    """Key splits for one forward launch over `rows` text rows.  A work-group
+    covers 128 (row, head) pairs of one kv head (4 waves x 32 rows); a one-round
+    launch (256 rows) has 64 of them on a 256-CU GPU, so the key range is cut
+    into up to 8 parts (each at least 512 keys) until there are two work-groups
+    per CU; the parts are folded by the merge kernel."""
+    hg = math.gcd(Hq // Hkv, 4)
+    wgs = B * (Hq // hg) * -(-rows // (32 * (4 // hg)))
+    s = 1
+    while s < 8 and wgs * s < target_wgs and Lkv // (2 * s) >= 512:
+        s *= 2
+    return s
+
+
 def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
                   local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
                   rounds: Optional[int] = None, mask: Optional[Mask] = None,
                   acc_in: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                  kv_splits: int = 1, batched: bool = False):
+                  kv_splits: Optional[int] = None, batched: bool = False):
     """Returns (q, k, v, o, L) like the reference (attn.py:435): o [B,Hq,Lq,D]
     bf16, L [B*Hq, Lq] fp32 natural-log LSE of sm_scale * q k^T.
 
@@ -65,7 +80,8 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     Keyword-only additions: `rounds` (P; default the size set by
     initialize_distributed), `mask`, `acc_in` = (O_in bf16 [B,Hq,Lq,D],
     L_in fp32 [B*Hq,Lq]) for every block, `kv_splits` (key ranges per round
-    computed by separate work-groups), `batched` (one launch over all P blocks
+    computed by separate work-groups; default: enough to give every CU two
+    work-groups, see auto_kv_splits), `batched` (one launch over all P blocks
     instead of one per round)."""
     _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
     q_, k_, v_ = _usable(q), _usable(k), _usable(v)
@@ -84,6 +100,8 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
     max_rows = max(r1 - r0 for r0, r1 in windows)
+    if kv_splits is None:
+        kv_splits = auto_kv_splits(B, Hq, k_.shape[1], max_rows, k_.shape[2])
     ws = None
     if kv_splits > 1:
         nbytes = ops.fwd_workspace_bytes(q_, k_, max_rows, kv_splits)

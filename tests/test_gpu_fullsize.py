@@ -40,14 +40,18 @@ def test_cfg1_forward_full_size(lvx):
     w = orc.make_inputs(orc.workload("cfg1"), need_grad_inputs=False)
     t = w.tensors
     q, k, v = _dev(t["q"]), _dev(t["k"]), _dev(t["v"])
-    _, _, _, o_r, l_r = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds)
+    _, _, _, o_r, l_r = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, kv_splits=1)
     _, _, _, o_b, l_b = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, batched=True)
     _, _, _, o_s, l_s = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, kv_splits=4)
     torch.cuda.synchronize()
     # one launch over all 16 blocks computes exactly what 16 launches compute
     assert torch.equal(o_r, o_b) and torch.equal(l_r, l_b)
-    # 4 key splits folded by the merge kernel: same result to bf16 rounding
+    # 4 key splits folded by the merge kernel: same result to bf16 rounding; so is the
+    # default (key splits chosen per launch size)
     assert (o_r.float() - o_s.float()).abs().max() <= 2e-2 and (l_r - l_s).abs().max() <= 1e-3
+    _, _, _, o_a, l_a = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds)
+    torch.cuda.synchronize()
+    assert (o_r.float() - o_a.float()).abs().max() <= 2e-2 and (l_r - l_a).abs().max() <= 1e-3
     # oracle on kv heads 0 and 5 (q heads 0-3 and 20-23), all rows, all keys
     for hk in (0, 5):
         hs = slice(4 * hk, 4 * hk + 4)
