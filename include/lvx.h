@@ -57,6 +57,14 @@ typedef struct lvx_attn_shape {
     const int32_t* kv_len;   /* [B] valid visual tokens per sample, or NULL */
     const int32_t* kv_start; /* [B, Lq] first visible token per text row, or NULL */
     const int32_t* kv_end;   /* [B, Lq] one past the last visible token (both or neither) */
+    /* Dense additive bias, fp32, added to scale * q k^T before the softmax (the tensor the
+     * reference's bias_func returns, lv_xattn/attn.py:386-389, 238-241), or NULL.  Element
+     * (b, h, row, key) is at bias[b*bias_stride_b + h*bias_stride_h + row*bias_stride_r + key];
+     * bias_stride_h = 0 broadcasts over heads.  -inf entries mask.  No gradient is formed
+     * for it (the reference forms none).  Rows are read in groups of 4 keys, so
+     * bias_stride_r must be at least Lkv rounded up to a multiple of 4 (pad the rows). */
+    const float* bias;
+    int64_t bias_stride_b, bias_stride_h, bias_stride_r;
 } lvx_attn_shape;
 
 /* A 4-d tensor with unit last stride. */

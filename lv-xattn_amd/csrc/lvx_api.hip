@@ -27,6 +27,11 @@ int check_shape(const lvx_attn_shape* s) {
     if (s->Hq % s->Hkv) return LVX_ERR_SHAPE;
     if (!(s->scale > 0.f) || !std::isfinite(s->scale)) return LVX_ERR_SCALE;
     if ((s->kv_start == nullptr) != (s->kv_end == nullptr)) return LVX_ERR_NULL;
+    if (s->bias) {
+        if (reinterpret_cast<uintptr_t>(s->bias) & 3) return LVX_ERR_ALIGN;
+        // rows are read in groups of 4 keys: a row must be readable up to Lkv rounded up to 4
+        if (s->bias_stride_r < (s->Lkv + 3) / 4 * 4) return LVX_ERR_SHAPE;
+    }
     return LVX_OK;
 }
 
@@ -100,6 +105,7 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.v = static_cast<const uint16_t*>(v->ptr);
     p.qs = st3(q); p.ks = st3(k); p.vs = st3(v);
     p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
+    p.bias = s->bias; p.bias_b = s->bias_stride_b; p.bias_h = s->bias_stride_h; p.bias_r = s->bias_stride_r;
     p.B = s->B; p.Hq = s->Hq; p.Hkv = s->Hkv; p.Lq = s->Lq; p.Lkv = s->Lkv;
     p.G = s->Hq / s->Hkv;
     p.HG = gcd(p.G, 4);
@@ -268,6 +274,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.dk = dk->ptr; p.dv = dv->ptr;
     p.qs = st3(q); p.ks = st3(k); p.vs = st3(v); p.dos = st3(dout); p.dks = st3(dk); p.dvs = st3(dv);
     p.kv_len = s->kv_len; p.kv_start = s->kv_start; p.kv_end = s->kv_end;
+    p.bias = s->bias; p.bias_b = s->bias_stride_b; p.bias_h = s->bias_stride_h; p.bias_r = s->bias_stride_r;
     p.B = s->B; p.Hq = s->Hq; p.Hkv = s->Hkv; p.Lq = s->Lq; p.Lkv = s->Lkv; p.G = s->Hq / s->Hkv;
     p.row_begin = row_begin; p.row_end = row_begin + row_count;
     p.n_kv_blocks = (s->Lkv + 127) / 128;

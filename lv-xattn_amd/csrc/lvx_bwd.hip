@@ -67,7 +67,8 @@ constexpr int SMEM_ELEMS = LOOP_ELEMS > EPI_ELEMS ? LOOP_ELEMS : EPI_ELEMS;
 
 constexpr float LOG2E = 1.4426950408889634f;
 
-template <bool MASKED>
+// BIAS: a dense fp32 bias joins the exponent, P = exp2(S*c + bias*log2e - LSE*log2e).
+template <bool MASKED, bool BIAS>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
     // per-row metadata of a staged tile, one per tile buffer: 8 x 16 bytes each of
@@ -205,8 +206,16 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // Flags say which halves exist at the edges of the walk; they are compile-time
     // constants in the steady-state loop.
     auto p_step = [&](auto tail_c, bool s_live, bool pv_live, const uint16_t* tile_cur, const uint16_t* tile_prev,
-                      const u32x4* meta, uint16_t* pbuf, f32x16& s_carry) __attribute__((always_inline)) {
+                      const u32x4* meta, uint16_t* pbuf, f32x16& s_carry, int64_t bias_off, int bias_r0)
+                      __attribute__((always_inline)) {
         constexpr bool TAIL = decltype(tail_c)::value;
+        float bv[16];
+        if (BIAS && pv_live) {   // bias of (row 8 vg + 4 g + r of the previous tile, this lane's token)
+            const float* bp = p.bias + bias_off + min(my_kv, p.Lkv - 1);
+            const int last = p.row_end - 1 - bias_r0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) bv[v] = bp[(int64_t)min(8 * (v >> 2) + 4 * g + (v & 3), last) * p.bias_r];
+        }
         const char* qt = reinterpret_cast<const char*>(tile_cur);
         const char* dot = reinterpret_cast<const char*>(tile_prev) + TILE_ELEMS * 2;
         bf16x8 qa[8];
@@ -239,7 +248,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             for (int vg = 0; vg < 4; ++vg) {
                 const f32x4 l4 = __builtin_bit_cast(f32x4, meta[2 * vg + g]);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) s[4 * vg + r] = __builtin_amdgcn_exp2f(fmaf(s[4 * vg + r], c, -l4[r]));
+                for (int r = 0; r < 4; ++r) {
+                    const float off = BIAS ? fmaf(bv[4 * vg + r], LOG2E, -l4[r]) : -l4[r];
+                    s[4 * vg + r] = __builtin_amdgcn_exp2f(fmaf(s[4 * vg + r], c, off));
+                }
             }
             if (MASKED) {
 #pragma unroll
@@ -351,14 +363,23 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // dS^T workspace offsets of the tiles in flight: a tile enters at [5] when requested
         // (two steps ahead); at step i (before that step's shift) tile i is at [3], tile i-3 at [0]
         int64_t w_q[6] = {0, 0, 0, 0, 0, 0};
+        int64_t b_q[6] = {0, 0, 0, 0, 0, 0};    // BIAS: offset of (b, h, first row of the tile) in the bias
+        int r_q[6] = {0, 0, 0, 0, 0, 0};        // BIAS: first row of the tile
         auto fetch = [&](int buf) {   // start the loads of the next tile of the walk
             w_q[5] = ws_head + (int64_t)cur_qt * (BN * BM);
+            if (BIAS) {
+                r_q[5] = p.row_begin + cur_qt * BM;
+                b_q[5] = b * p.bias_b + (hk * p.G + cur_gi) * p.bias_h + (int64_t)r_q[5] * p.bias_r;
+            }
             prefetch(buf);
             advance();
         };
         auto shift = [&]() {
 #pragma unroll
-            for (int k = 0; k < 5; ++k) w_q[k] = w_q[k + 1];
+            for (int k = 0; k < 5; ++k) {
+                w_q[k] = w_q[k + 1];
+                if (BIAS) { b_q[k] = b_q[k + 1]; r_q[k] = r_q[k + 1]; }
+            }
         };
         f32x16 carry;     // P-wave: raw S of the previous tile; D-wave: dP of the previous tile
 #pragma unroll
@@ -377,7 +398,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             if (i + 2 < n_iter) fetch(m5(rc + 2));
             const int r1 = m5(rc + 4), r2 = m5(rc + 3);     // (i - 1) % 5, (i - 2) % 5
             if (!DROLE)
-                p_step(tail_c, s_live, pv_live, qd(rc), qd(r1), meta_s4[r1], pbf((i + 1) & 1), carry);
+                p_step(tail_c, s_live, pv_live, qd(rc), qd(r1), meta_s4[r1], pbf((i + 1) & 1), carry, b_q[2], r_q[2]);
             else
                 d_step(pv_live, ds_live, qd(r1), qd(r2), meta_s4[r2], pbf(i & 1), dst(i & 1), carry);
             // dS^T(i-3) to HBM last: its LDS read queues behind this step's operand reads
@@ -466,10 +487,13 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
-    if (masked)
-        hipLaunchKernelGGL(bwd_kernel<true>, dim3(grid), dim3(NT), 0, st, p);
-    else
-        hipLaunchKernelGGL(bwd_kernel<false>, dim3(grid), dim3(NT), 0, st, p);
+    if (p.bias) {
+        if (masked) hipLaunchKernelGGL((bwd_kernel<true, true>), dim3(grid), dim3(NT), 0, st, p);
+        else hipLaunchKernelGGL((bwd_kernel<false, true>), dim3(grid), dim3(NT), 0, st, p);
+    } else {
+        if (masked) hipLaunchKernelGGL((bwd_kernel<true, false>), dim3(grid), dim3(NT), 0, st, p);
+        else hipLaunchKernelGGL((bwd_kernel<false, false>), dim3(grid), dim3(NT), 0, st, p);
+    }
     return hipGetLastError();
 }
 

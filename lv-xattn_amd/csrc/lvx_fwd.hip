@@ -40,8 +40,11 @@ constexpr int BN = 64;        // keys per tile
 constexpr int TILE_BYTES = BN * D * 2;
 constexpr int BIG = 0x3fffffff;
 constexpr float RESCALE_LOG2 = 8.f;
+constexpr float LOG2E_F = 1.4426950408889634f, LN2_F = 0.6931471805599453f;
 
-template <bool MASKED>
+// BIAS: a dense fp32 bias is added to scale * S before the softmax; the scores are
+// then carried in log2 units (S*c + bias*log2e) instead of raw.
+template <bool MASKED, bool BIAS>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
@@ -158,6 +161,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
     const float c = p.scale_log2e;
+    const float cc = BIAS ? 1.f : c;              // factor from the carried scores to log2 units
+    const float* brow = nullptr;                  // this lane's row of the bias
+    if (BIAS) brow = p.bias + b * p.bias_b + h * p.bias_h + (int64_t)min(row, p.row_end - 1) * p.bias_r;
 
     const int t_begin = (hi > lo) ? lo / BN : 0;
     const int t_end = (hi > lo) ? (hi + BN - 1) / BN : 0;
@@ -207,6 +213,22 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
             }
         __builtin_amdgcn_sched_barrier(0);
 
+        if (BIAS) {
+            // register group vg of lane-half g holds keys kv0 + 8 vg + 4 g + 0..3 (+32 for s1);
+            // groups past the end re-read the last one (those keys are masked below)
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                const int k0 = kv0 + 8 * vg + 4 * g;
+                const f32x4 ba = *reinterpret_cast<const f32x4*>(brow + min(k0, (p.Lkv - 1) & ~3));
+                const f32x4 bb = *reinterpret_cast<const f32x4*>(brow + min(k0 + 32, (p.Lkv - 1) & ~3));
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    s0[4 * vg + r] = fmaf(s0[4 * vg + r], c, ba[r] * LOG2E_F);
+                    s1[4 * vg + r] = fmaf(s1[4 * vg + r], c, bb[r] * LOG2E_F);
+                }
+            }
+        }
+
         if (kv0 < in_lo || kv0 + BN > in_hi) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -229,12 +251,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         // maximum has grown by more than 2^RESCALE_LOG2 since it was set, so P may
         // reach 2^RESCALE_LOG2 instead of 1 (harmless in fp32 / bf16) and the
         // rescale of O happens a few times per row instead of almost every tile.
-        const float mcand = mx * c;                       // mx >= m_i
-        const float m_ic = m_i * c;
+        const float mcand = mx * cc;                      // mx >= m_i
+        const float m_ic = m_i * cc;
         const bool move = (mx != -INFINITY) && !(mcand - m_ic <= RESCALE_LOG2);
         const float alpha = move ? __builtin_amdgcn_exp2f(m_ic - mcand) : 1.f;
         if (move) m_i = mx;
-        const float mc = (m_i == -INFINITY) ? 0.f : m_i * c;
+        const float mc = (m_i == -INFINITY) ? 0.f : m_i * cc;
 
         // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile.  The row
         // sum is taken in fp32 before the rounding to bf16 (summing the rounded
@@ -247,8 +269,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int v = 8 * j + 2 * e;
-                const float a0 = __builtin_amdgcn_exp2f(fmaf(s0[v], c, -mc)), a1 = __builtin_amdgcn_exp2f(fmaf(s0[v + 1], c, -mc));
-                const float b0 = __builtin_amdgcn_exp2f(fmaf(s1[v], c, -mc)), b1 = __builtin_amdgcn_exp2f(fmaf(s1[v + 1], c, -mc));
+                const float a0 = __builtin_amdgcn_exp2f(fmaf(s0[v], cc, -mc)), a1 = __builtin_amdgcn_exp2f(fmaf(s0[v + 1], cc, -mc));
+                const float b0 = __builtin_amdgcn_exp2f(fmaf(s1[v], cc, -mc)), b1 = __builtin_amdgcn_exp2f(fmaf(s1[v + 1], cc, -mc));
                 rs0 += a0 + a1;
                 rs1 += b0 + b1;
                 u0[e] = pack_bf16(a0, a1);
@@ -292,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
                 *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * vg + 4 * g) = w;
             }
         if (g == 0) {
-            const float lse = l_tot > 0.f ? m_i * p.scale + __logf(l_tot) : -INFINITY;
+            const float lse = l_tot > 0.f ? m_i * (BIAS ? LN2_F : p.scale) + __logf(l_tot) : -INFINITY;
             p.lse[split * p.lse_split_stride + ((int64_t)b * p.Hq + h) * p.lse_bh_stride + row] = lse;
         }
     }
@@ -302,10 +324,13 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
-    if (masked)
-        hipLaunchKernelGGL(fwd_kernel<true>, dim3(grid), dim3(256), 0, st, p);
-    else
-        hipLaunchKernelGGL(fwd_kernel<false>, dim3(grid), dim3(256), 0, st, p);
+    if (p.bias) {
+        if (masked) hipLaunchKernelGGL((fwd_kernel<true, true>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((fwd_kernel<false, true>), dim3(grid), dim3(256), 0, st, p);
+    } else {
+        if (masked) hipLaunchKernelGGL((fwd_kernel<true, false>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((fwd_kernel<false, false>), dim3(grid), dim3(256), 0, st, p);
+    }
     return hipGetLastError();
 }
 

@@ -23,6 +23,8 @@ struct FwdParams {
     const int32_t* kv_len;
     const int32_t* kv_start;
     const int32_t* kv_end;
+    const float* bias;         // dense additive bias or nullptr; element strides below
+    int64_t bias_b, bias_h, bias_r;
     int B, Hq, Hkv, Lq, Lkv;
     int G;                     // q heads per kv head
     int HG;                    // q heads a work-group covers (one per wave)
@@ -69,6 +71,8 @@ struct BwdParams {
     const int32_t* kv_len;
     const int32_t* kv_start;
     const int32_t* kv_end;
+    const float* bias;         // dense additive bias or nullptr; element strides below
+    int64_t bias_b, bias_h, bias_r;
     int B, Hq, Hkv, Lq, Lkv, G;
     int row_begin, row_end;
     int n_kv_blocks, total_wg;
@@ -130,7 +134,7 @@ struct GemmParams {
     int a_tiled_m;
 };
 
-hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st);
+hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st);   // p.bias selects the bias variant
 hipError_t launch_merge(const MergeParams& p, hipStream_t st);
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st);
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);

@@ -26,6 +26,7 @@ class AttnShape(C.Structure):
         ("B", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
         ("Lq", C.c_int32), ("Lkv", C.c_int32), ("dtype", C.c_int32), ("scale", C.c_float),
         ("kv_len", C.c_void_p), ("kv_start", C.c_void_p), ("kv_end", C.c_void_p),
+        ("bias", C.c_void_p), ("bias_stride_b", C.c_int64), ("bias_stride_h", C.c_int64), ("bias_stride_r", C.c_int64),
     ]
 
 

@@ -41,15 +41,33 @@ def _usable(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
-def _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args):
+def _reject_unsupported(causal):
     if causal:
         # the reference applies the triangle to rank-local indices only
         # (lv_xattn/attn.py:229,237), which means nothing once blocks travel
         raise ValueError("causal=True is not defined for cross-attention over travelling query blocks")
-    if bias_func is not None or len(local_bias_args) or len(remote_bias_args):
-        raise NotImplementedError(
-            "dense additive bias_func is not implemented on the gfx950 path; "
-            "pass the compact interval form via mask=Mask(kv_len, kv_start, kv_end)")
+
+
+def _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, dev) -> Optional[torch.Tensor]:
+    """The additive bias of the reference (lv_xattn/attn.py:386-389): there,
+    bias_func(*(local_bias_args + remote_bias_args)) is evaluated once per round
+    with the visiting block's remote arguments and yields [B, 1, Lb, Lkv].  Here
+    q holds all P blocks, so the remote arguments describe all Lq rows and the
+    one call yields [B|1, 1|Hq, Lq, Lkv]; every launch indexes it by absolute row."""
+    if bias_func is None:
+        if len(local_bias_args) or len(remote_bias_args):
+            raise ValueError("bias arguments given without a bias_func")
+        return None
+    bias = bias_func(*(list(local_bias_args) + list(remote_bias_args)))
+    if bias.dim() != 4 or tuple(bias.shape[2:]) != (Lq, Lkv) or bias.shape[0] not in (1, B) or bias.shape[1] not in (1, Hq):
+        raise ValueError(f"bias_func must return [B|1, 1|Hq, {Lq}, {Lkv}], got {tuple(bias.shape)}")
+    bias = bias.to(device=dev, dtype=torch.float32)
+    pad = -Lkv % 4          # the kernels read a row in groups of 4 keys
+    if bias.stride(3) != 1 or bias.stride(2) < Lkv + pad:
+        padded = torch.zeros(*bias.shape[:3], Lkv + pad, dtype=torch.float32, device=dev)
+        padded[..., :Lkv] = bias
+        bias = padded[..., :Lkv]
+    return bias
 
 
 def auto_kv_splits(B: int, Hq: int, Hkv: int, rows: int, Lkv: int, target_wgs: int = 512) -> int:
@@ -83,11 +101,12 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     computed by separate work-groups; default: enough to give every CU two
     work-groups, see auto_kv_splits), `batched` (one launch over all P blocks
     instead of one per round)."""
-    _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
+    _reject_unsupported(causal)
     q_, k_, v_ = _usable(q), _usable(k), _usable(v)
     B, Hq, Lq, D = q_.shape
     P = rounds if rounds is not None else get_sequence_parallel_size()
     dev = q_.device
+    bias = _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, k_.shape[2], dev)
     if mask is not None:
         mask = mask.to(dev)
 
@@ -110,12 +129,12 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     if acc_in is None:
         # merging into the identity returns the partial itself: write in place
         for r0, r1 in windows:
-            ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws)
+            ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
     else:
         o_part = workspace("fwd_o_part", (B, Hq, Lq, D), q_.dtype, dev)
         l_part = workspace("fwd_l_part", (B * Hq, Lq), torch.float32, dev)
         for r0, r1 in windows:
-            ops.fwd(q_, k_, v_, o_part, l_part, sm_scale, r0, r1 - r0, mask, kv_splits, ws)
+            ops.fwd(q_, k_, v_, o_part, l_part, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
             ops.merge(o, L, o_part, l_part, r0, r1 - r0)
     return q, k, v, o, L
 
@@ -131,12 +150,13 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     a group and across rounds and rounded to bf16 once; a round's dQ rows are
     complete after that round (fp32 sum over all local tokens, rounded once).
     `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored."""
-    _reject_unsupported(causal, bias_func, local_bias_args, remote_bias_args)
+    _reject_unsupported(causal)
     q_, k_, v_, o_, do_ = (_usable(t) for t in (q, k, v, o, do))
     B, Hq, Lq, D = q_.shape
     Hkv, Lkv = k_.shape[1], k_.shape[2]
     P = rounds if rounds is not None else get_sequence_parallel_size()
     dev = q_.device
+    bias = _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, dev)
     if mask is not None:
         mask = mask.to(dev)
     L_ = L.to(torch.float32).reshape(B * Hq, Lq).contiguous()
@@ -153,7 +173,7 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
         r0, r1 = windows[0]
         ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
         ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk, dv, sm_scale, r0, r1 - r0, mask, accumulate_dkv=False,
-                workspace=ws)
+                workspace=ws, bias=bias)
     else:
         dk_acc = workspace("bwd_dk_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
         dv_acc = workspace("bwd_dv_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
@@ -162,7 +182,7 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
         for r0, r1 in windows:
             ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
             ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
-                    accumulate_dkv=True, workspace=ws)
+                    accumulate_dkv=True, workspace=ws, bias=bias)
         # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
         ops.cast_f32_bf16(dk_acc.transpose(1, 2), dk.transpose(1, 2))
         ops.cast_f32_bf16(dv_acc.transpose(1, 2), dv.transpose(1, 2))

@@ -36,14 +36,19 @@ def create_attention_class_save_qkv(attention_mode: str = "lv_xattn", no_overlap
             q, k, v, o, L = _attn_forward(q, k, v, causal, sm_scale, None, bias_func, local_bias_args,
                                           remote_bias_args, no_overlap, rounds=rounds, mask=mask,
                                           batched=batched)
-            ctx.save_for_backward(q, k, v, o, L)
+            # like the reference (test_llama3.py:144-149): the bias arguments are kept and the
+            # bias is rebuilt in backward
+            ctx.save_for_backward(q, k, v, o, L, *local_bias_args, *remote_bias_args)
+            ctx.n_local = len(local_bias_args)
+            ctx.bias_func = bias_func
             ctx.sm_scale, ctx.causal, ctx.mask = sm_scale, causal, mask
             return o
 
         @staticmethod
         def backward(ctx, do):
-            q, k, v, o, L = ctx.saved_tensors
+            q, k, v, o, L, *bias_args = ctx.saved_tensors
             dq, dk, dv = _attn_backward(do, q, k, v, o, L, ctx.causal, ctx.sm_scale, None, "flash",
+                                        ctx.bias_func, bias_args[:ctx.n_local], bias_args[ctx.n_local:],
                                         no_overlap=no_overlap, rounds=rounds, mask=ctx.mask, batched=batched)
             return dq, dk, dv, None, None, None, None, None, None
 

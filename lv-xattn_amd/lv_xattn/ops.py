@@ -33,7 +33,8 @@ class Mask:
         return Mask(f(self.kv_len), f(self.kv_start), f(self.kv_end))
 
 
-def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask]) -> AttnShape:
+def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask],
+           bias: Optional[torch.Tensor] = None) -> AttnShape:
     if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16:
         raise LvxError(f"bf16 tensors required, got {q.dtype} / {k.dtype}")
     B, Hq, Lq, D = q.shape
@@ -50,6 +51,16 @@ def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask])
             if t.dtype != torch.int32 or tuple(t.shape) != want or not t.is_contiguous() or t.device != q.device:
                 raise LvxError(f"mask.{name} must be a contiguous int32 {want} tensor on {q.device}")
             setattr(s, name, t.data_ptr())
+    if bias is not None:
+        if (bias.dtype != torch.float32 or bias.dim() != 4 or bias.device != q.device or bias.stride(3) != 1
+                or bias.shape[0] not in (1, B) or bias.shape[1] not in (1, Hq) or tuple(bias.shape[2:]) != (Lq, Lkv)):
+            raise LvxError(f"bias must be an fp32 [B|1, Hq|1, {Lq}, {Lkv}] tensor with unit last stride on {q.device}")
+        if bias.stride(2) < (Lkv + 3) // 4 * 4:
+            raise LvxError("bias rows must be padded to a multiple of 4 floats (row stride >= Lkv rounded up to 4)")
+        s.bias = bias.data_ptr()
+        s.bias_stride_b = bias.stride(0) if bias.shape[0] > 1 else 0
+        s.bias_stride_h = bias.stride(1) if bias.shape[1] > 1 else 0
+        s.bias_stride_r = bias.stride(2)
     return s
 
 
@@ -59,10 +70,11 @@ def fwd_workspace_bytes(q, k, row_count: int, kv_splits: int) -> int:
 
 
 def fwd(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask] = None,
-        kv_splits: int = 1, workspace: Optional[torch.Tensor] = None) -> None:
+        kv_splits: int = 1, workspace: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
     """Partial O (bf16) and LSE (fp32 [B*Hq, Lq]) of text rows
-    [row_begin, row_begin+row_count) against the whole local K/V shard."""
-    s = _shape(q, k, scale, mask)
+    [row_begin, row_begin+row_count) against the whole local K/V shard.
+    `bias`: dense additive fp32 [B|1, Hq|1, Lq, Lkv], added after the scale."""
+    s = _shape(q, k, scale, mask, bias)
     if row_count is None:
         row_count = q.shape[2] - row_begin
     _check_lse(lse, q)
@@ -103,11 +115,12 @@ def bwd_workspace_bytes(q, k, row_count: int) -> int:
 
 def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=None,
         mask: Optional[Mask] = None, accumulate_dkv: bool = False,
-        workspace: Optional[torch.Tensor] = None) -> None:
+        workspace: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
     """Writes dq (bf16) for the selected rows and writes (bf16) or accumulates
     (fp32) dk, dv at Hkv heads.  `workspace`: uint8 tensor of at least
-    bwd_workspace_bytes(q, k, row_count) bytes."""
-    s = _shape(q, k, scale, mask)
+    bwd_workspace_bytes(q, k, row_count) bytes.  `bias` as in fwd (no gradient
+    is formed for it)."""
+    s = _shape(q, k, scale, mask, bias)
     if row_count is None:
         row_count = q.shape[2] - row_begin
     _check_lse(lse, q)

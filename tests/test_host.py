@@ -44,13 +44,15 @@ def test_workspace_cache_and_reset():
     lv_xattn.reset_global_memory_buffer("lv_xattn")      # the reference passes the mode
 
 
-def test_causal_and_bias_are_rejected_explicitly():
+def test_causal_and_malformed_bias_are_rejected_explicitly():
     q = torch.zeros(1, 4, 8, 128, dtype=torch.bfloat16)
     k = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="causal"):
         lv_xattn._attn_forward(q, k, k, True, 0.1, None)
-    with pytest.raises(NotImplementedError, match="bias_func"):
-        lv_xattn._attn_forward(q, k, k, False, 0.1, None, bias_func=lambda: None)
+    with pytest.raises(ValueError, match="bias_func must return"):
+        lv_xattn._attn_forward(q, k, k, False, 0.1, None, bias_func=lambda: torch.zeros(1, 1, 3, 8))
+    with pytest.raises(ValueError, match="without a bias_func"):
+        lv_xattn._attn_forward(q, k, k, False, 0.1, None, local_bias_args=[torch.zeros(1)])
     with pytest.raises(ValueError, match="causal"):
         lv_xattn._attn_backward(q, q, k, k, q, torch.zeros(4, 8), True, 0.1, None, "flash")
 

@@ -279,3 +279,27 @@ def test_layer_reference_small_gradients_vs_autograd():
     for a, b in ((out["dq"], gq), (out["dk"], gk), (out["dv"], gv)):
         rel = (a.double() - b).norm() / b.norm()
         assert rel < 5e-3
+
+
+def test_backward_with_bias_against_autograd():
+    # additive bias (with -inf entries) enters P = softmax(scale*S + bias) and gets no
+    # gradient: compare the hand-written backward with autograd through the dense formula
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(1, 4, 10, 16, generator=g).double().requires_grad_()
+    k = torch.randn(1, 2, 14, 16, generator=g).double().requires_grad_()
+    v = torch.randn(1, 2, 14, 16, generator=g).double().requires_grad_()
+    do = torch.randn(1, 4, 10, 16, generator=g).double()
+    bias = torch.randn(1, 1, 10, 14, generator=g).double()
+    bias[0, 0, :, 3] = float("-inf")
+    bias[0, 0, 2, :7] = float("-inf")
+    ke, ve = k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1)
+    s = 0.3 * q @ ke.transpose(-1, -2) + bias
+    o = torch.softmax(s, -1) @ ve
+    o.backward(do)
+    o_r, lse = orc.attention_dense(q.detach().float(), k.detach().float(), v.detach().float(), 0.3, bias=bias.float())
+    dq, dk, dv = orc.attention_backward(do.float(), q.detach().float(), k.detach().float(), v.detach().float(),
+                                        o_r, lse, 0.3, bias=bias.float(), rounds=2)
+    assert (o_r.double() - o.detach()).abs().max() < 1e-5
+    assert (dq.double() - q.grad).abs().max() < 1e-4
+    assert (dk.double() - k.grad).abs().max() < 1e-4
+    assert (dv.double() - v.grad).abs().max() < 1e-4
