@@ -62,7 +62,9 @@ typedef struct lvx_attn_shape {
      * (b, h, row, key) is at bias[b*bias_stride_b + h*bias_stride_h + row*bias_stride_r + key];
      * bias_stride_h = 0 broadcasts over heads.  -inf entries mask.  No gradient is formed
      * for it (the reference forms none).  Rows are read in groups of 4 keys, so
-     * bias_stride_r must be at least Lkv rounded up to a multiple of 4 (pad the rows). */
+     * bias_stride_r must be at least Lkv rounded up to a multiple of 4 (pad the rows).
+     * Mask with -inf or a moderate negative (e.g. -30000), not with -FLT_MAX-sized values:
+     * the backward subtracts the row's LSE from score + bias in fp32. */
     const float* bias;
     int64_t bias_stride_b, bias_stride_h, bias_stride_r;
 } lvx_attn_shape;

@@ -1,0 +1,75 @@
+"""Hugging Face integration for Llama-3.2-Vision (Mllama) cross-attention.
+
+The reference replaces `MllamaTextCrossSdpaAttention.forward` of transformers
+4.47 by hand (test_llama3.py:356-468, installed at :666-668).  Current
+transformers releases route every attention layer through a pluggable
+attention interface, so the same substitution is one registration:
+
+    from lv_xattn.hf_mllama import register
+    register()                                  # adds the "lv_xattn" implementation
+    model.config._attn_implementation = "lv_xattn"      # or per sub-config
+
+`MllamaTextCrossAttention.forward` then hands the projected, normalised
+Q [B,Hq,Lq,D], K, V [B,Hkv,Lkv,D] and the additive cross-attention mask
+[B,1,Lq,Lkv] to `lv_xattn_attention_forward`, which runs the gfx950 flash
+forward / backward (dense-bias variant; K/V kept for backward, as in the
+reference's `create_attention_class_save_qkv`, test_llama3.py:125-178).
+Self-attention layers and anything the kernels do not cover (head_dim other
+than 128, dropout, a causal request) fall back to transformers' eager path.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .autograd import create_attention_class_save_qkv
+
+NAME = "lv_xattn"
+_attention = None
+
+
+def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
+    """transformers fills masked positions with the dtype's most negative finite
+    value (-3.4e38 in bf16).  The kernels add the bias to the fp32 scores and, in
+    backward, subtract the row's LSE from score + bias, so the fill value is
+    limited to -30000: exp(-30000) is still exactly 0 next to any visible key,
+    and the subtraction stays accurate.  A row that is masked everywhere then
+    attends by its scores over the masked keys (as it does in the reference,
+    whose fp16 fill value is -65504; transformers' eager path attends uniformly
+    there) - the Mllama decoder layer zeroes such rows right after the
+    attention (full_text_row_masked_out_mask), so the difference never shows."""
+    return mask.float().clamp_min(-30000.0)
+
+
+def lv_xattn_attention_forward(module, query, key, value, attention_mask: Optional[torch.Tensor],
+                               dropout: float = 0.0, scaling: Optional[float] = None, **kwargs):
+    """Attention-interface function (same contract as transformers'
+    eager_attention_forward): returns (attn_output [B, Lq, Hq, D], None)."""
+    global _attention
+    usable = (query.is_cuda and query.dtype == torch.bfloat16 and query.shape[-1] == 128 and dropout == 0.0
+              and not kwargs.get("is_causal", False) and getattr(module, "is_causal", False) is not True
+              and query.shape[1] % key.shape[1] == 0)
+    if not usable:
+        from transformers.models.mllama.modeling_mllama import eager_attention_forward
+        return eager_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
+                                       scaling=scaling, **kwargs)
+    if _attention is None:
+        _attention = create_attention_class_save_qkv("lv_xattn", rounds=1, batched=True).apply
+    if scaling is None:
+        scaling = query.shape[-1] ** -0.5
+    if attention_mask is None:
+        out = _attention(query, key, value, False, scaling)
+    else:
+        Lq, Lkv = query.shape[2], key.shape[2]
+        mask = attention_mask[..., :Lq, :Lkv]
+        out = _attention(query, key, value, False, scaling, _mask_bias, [mask], [])
+    return out.transpose(1, 2).contiguous(), None
+
+
+def register() -> str:
+    """Adds the implementation to transformers' attention registry and returns
+    its name.  Raises ImportError if transformers has no attention interface."""
+    from transformers import AttentionInterface
+    AttentionInterface.register(NAME, lv_xattn_attention_forward)
+    return NAME
