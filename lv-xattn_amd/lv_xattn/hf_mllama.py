@@ -73,3 +73,36 @@ def register() -> str:
     from transformers import AttentionInterface
     AttentionInterface.register(NAME, lv_xattn_attention_forward)
     return NAME
+
+
+def mask_from_cross_attention_mask(cross_attention_mask: torch.Tensor, num_vision_tokens: int,
+                                   kv_len: Optional[torch.Tensor] = None):
+    """Compact form of a Llama-3.2 cross-attention mask.
+
+    `cross_attention_mask` is what the Mllama processor emits, [B, T, n_images,
+    n_tiles] with 1 where text token t may look at that tile; every tile stands
+    for `num_vision_tokens` consecutive keys, in (image, tile) order - the
+    expansion transformers does in `_prepare_cross_attention_mask` before
+    turning it into the dense additive bias the reference feeds to `bias_func`
+    (lv_xattn/attn.py:386-389).  When every row's visible keys form one
+    contiguous range (the usual case: a token looks at the tiles of the most
+    recent image) this returns `Mask(kv_len, kv_start, kv_end)` for the interval
+    kernels - 8 bytes per row instead of 4 bytes per (row, key); rows that see
+    nothing get an empty interval (O = 0, LSE = -inf, dQ = 0).  Returns None if
+    some row has a gap (e.g. unused tile slots between two visible images): use
+    the dense bias then."""
+    from .ops import Mask
+    B, T = cross_attention_mask.shape[:2]
+    vis = cross_attention_mask.reshape(B, T, -1) != 0              # [B, T, n_images * n_tiles]
+    n = vis.shape[-1]
+    idx = torch.arange(n, device=vis.device)
+    any_vis = vis.any(-1)
+    first = torch.where(vis, idx, n).amin(-1)
+    last = torch.where(vis, idx, -1).amax(-1)
+    count = vis.sum(-1)
+    if not bool(((last - first + 1 == count) | ~any_vis).all()):
+        return None
+    start = torch.where(any_vis, first, torch.zeros_like(first)) * num_vision_tokens
+    end = torch.where(any_vis, last + 1, torch.zeros_like(last)) * num_vision_tokens
+    return Mask(None if kv_len is None else kv_len.to(torch.int32), start.to(torch.int32).contiguous(),
+                end.to(torch.int32).contiguous())

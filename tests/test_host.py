@@ -71,3 +71,24 @@ def test_shape_and_dtype_checks_raise_before_any_device_call():
         ops._shape(qb, kb, 0.1, bad)
     with pytest.raises(ops.LvxError, match="unit last stride"):
         ops.t4(torch.zeros(1, 2, 128, 8, dtype=torch.bfloat16).transpose(2, 3))
+
+
+def test_llama_cross_attention_mask_to_intervals():
+    from lv_xattn.hf_mllama import mask_from_cross_attention_mask
+    # 2 samples, 6 text tokens, 2 images x 4 tile slots, 5 keys per tile
+    cam = torch.zeros(2, 6, 2, 4, dtype=torch.int64)
+    cam[0, 1:4, 0, :2] = 1          # tokens 1-3 see tiles 0,1 of image 0
+    cam[0, 4:, 1, :] = 1            # tokens 4-5 see all four tiles of image 1
+    cam[1, 2:, 0, :4] = 1           # sample 1: tokens 2.. see image 0 (4 tiles) ...
+    cam[1, 5, 1, :1] = 1            # ... and token 5 also tile 0 of image 1 (adjacent: still one range)
+    m = mask_from_cross_attention_mask(cam, 5)
+    assert m is not None and m.kv_start.dtype == torch.int32
+    assert m.kv_start.tolist() == [[0, 0, 0, 0, 20, 20], [0, 0, 0, 0, 0, 0]]
+    assert m.kv_end.tolist() == [[0, 10, 10, 10, 40, 40], [0, 0, 20, 20, 20, 25]]
+    # the dense expansion transformers builds says the same
+    dense = cam.reshape(2, 6, 8).repeat_interleave(5, dim=-1).bool()
+    k = torch.arange(40)
+    assert torch.equal(dense, (k >= m.kv_start[..., None]) & (k < m.kv_end[..., None]))
+    # a gap (image 0 with 2 of 4 tiles, then image 1) has no interval form
+    cam[0, 5, 0, :2] = 1
+    assert mask_from_cross_attention_mask(cam, 5) is None
