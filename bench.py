@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes moved by one lvx_bwd call at cfg2 (zero + dK/dV kernel + 2 casts + dQ GEMM), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy (profiles/cfg2_bwd_hbm_traffic.md)
-BWD_TRAFFIC_BYTES = {"cfg2": 4.41e9}
+BWD_TRAFFIC_BYTES = {"cfg2": 4.48e9}
 
 
 def flops(w, n_pairs):
@@ -295,7 +295,7 @@ def main():
         kb = kernel_breakdown(layer, npairs, torch)
         out["kernels"] = kb
         dom = kb["bwd_all_rounds_one_launch"]
-        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = zero_kernel + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
+        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel + zero_kernel + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
                            "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
                            "traffic": BWD_TRAFFIC_BYTES.get(w.name) if a.mode == "batched" else None,
