@@ -117,10 +117,12 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const int n_iter = (kvb < kv_len) ? max(0, min(p.split_steps, p.G * n_qtiles - it_lo)) : 0;
     const float c = p.scale_log2e;
 
-    // global -> LDS: wave w moves rows 4w..4w+3 of the Q tile and of the dO tile
-    // (one 1 KiB load each); lane i fills position i & 15 of row 4w + (i >> 4).
-    const int ld_r = 4 * wave + (lane >> 4);
-    const uint32_t ld_c = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | (wave & 3))) * 16u;
+    // global -> LDS is the P-waves' job (their step is the shorter one): P-wave w moves
+    // rows 8w..8w+7 of the Q tile and of the dO tile as two 1 KiB loads each (4 rows
+    // per load); lane i fills position i & 15 of row 4 ch + (i >> 4), ch = 2w, 2w+1.
+    const int ld_r = 8 * slice + (lane >> 4);          // first of the two rows, the other is 4 further
+    const uint32_t ld_c0 = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice) & 3))) * 16u;
+    const uint32_t ld_c1 = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice + 1) & 3))) * 16u;
     const uint32_t qrow_b = (uint32_t)p.qs.s * 2u, dorow_b = (uint32_t)p.dos.s * 2u;   // bytes per text row
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t meta0 = (uint32_t)(uintptr_t)&meta_s4[0][0];
@@ -142,7 +144,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
     }
     const int pb_off = slice * (2 * 64 * 8) + lane * 8;
-    const int cp_token = tid >> 2, cp_part = tid & 3;
+    // dS^T copy-out, also by the P-waves: 512 chunks of 16 bytes, two per thread (tokens t >> 2 and 64 + (t >> 2))
+    const int cp_token = (tid & 255) >> 2, cp_part = tid & 3;
     // workspace tile (b, h, token block, row tile): [128 tokens][32 rows], 8 KB, contiguous
     uint16_t* ws_lane = p.ds_ws + (int64_t)kblk * p.ws_ld + cp_token * BM + cp_part * 8;
 
@@ -177,10 +180,13 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 dma4_addr(reinterpret_cast<const char*>(iv), mslot + 256);
             }
         }
-        const uint32_t row = (uint32_t)min(r0 + ld_r, p.row_end - 1);
-        const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)wave * 1024u;
-        dma16(q_head, row * qrow_b + ld_c, slot);
-        dma16(do_head, row * dorow_b + ld_c, slot + TILE_ELEMS * 2);
+        const uint32_t row0 = (uint32_t)min(r0 + ld_r, p.row_end - 1);
+        const uint32_t row1 = (uint32_t)min(r0 + ld_r + 4, p.row_end - 1);
+        const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)slice * 2048u;
+        dma16(q_head, row0 * qrow_b + ld_c0, slot);
+        dma16(q_head, row1 * qrow_b + ld_c1, slot + 1024);
+        dma16(do_head, row0 * dorow_b + ld_c0, slot + TILE_ELEMS * 2);
+        dma16(do_head, row1 * dorow_b + ld_c1, slot + TILE_ELEMS * 2 + 1024);
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
         if (++cur_qt == n_qtiles) {
@@ -192,7 +198,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     // the finished dS^T tile goes to HBM as one contiguous 8 KB block
     auto copy_out = [&](const uint16_t* dst, int64_t ws_off) {
-        *reinterpret_cast<u32x4*>(ws_lane + ws_off) = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
+        const u32x4 a = *reinterpret_cast<const u32x4*>(dst + cp_token * DSS + cp_part * 8);
+        const u32x4 c2 = *reinterpret_cast<const u32x4*>(dst + (cp_token + 64) * DSS + cp_part * 8);
+        *reinterpret_cast<u32x4*>(ws_lane + ws_off) = a;
+        *reinterpret_cast<u32x4*>(ws_lane + ws_off + 64 * BM) = c2;
     };
 
     // The work on a tile is spread over three steps so that, inside every wave, the
@@ -371,7 +380,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 r_q[5] = p.row_begin + cur_qt * BM;
                 b_q[5] = b * p.bias_b + (hk * p.G + cur_gi) * p.bias_h + (int64_t)r_q[5] * p.bias_r;
             }
-            prefetch(buf);
+            if (!DROLE) prefetch(buf);
             advance();
         };
         auto shift = [&]() {
@@ -387,12 +396,14 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         int rc = 0;       // i % 5
 
         auto step = [&](int i, bool s_live, bool pv_live, bool ds_live, bool copy) __attribute__((always_inline)) {
-            // This wave's part of tile i (requested two steps ago) must have landed.  When
-            // the previous step requested a tile, the wave has issued since: a dS^T store,
-            // [wave 0: metadata loads,] 2 tile loads, a store.  Loads complete in order, so
-            // "at most 2 operations outstanding" covers tile i and leaves tile i+1 in flight.
-            if (i + 1 < n_iter) wait_vmcnt<2>();
-            else wait_vmcnt<0>();
+            // A P-wave's part of tile i (requested two steps ago) must have landed.  When the
+            // previous step requested a tile, the wave has issued since: 2 dS^T stores,
+            // [wave 0: metadata loads,] 4 tile loads, 2 stores.  Loads complete in order, so
+            // "at most 4 operations outstanding" covers tile i and leaves tile i+1 in flight.
+            if (!DROLE) {
+                if (i + 1 < n_iter) wait_vmcnt<4>();
+                else wait_vmcnt<0>();
+            }
             lds_barrier();
             // tile i+2 replaces tile i-3, whose last readers finished before this barrier
             if (i + 2 < n_iter) fetch(m5(rc + 2));
@@ -403,7 +414,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 d_step(pv_live, ds_live, qd(r1), qd(r2), meta_s4[r2], pbf(i & 1), dst(i & 1), carry);
             // dS^T(i-3) to HBM last: its LDS read queues behind this step's operand reads
             // instead of delaying them, and only has to finish before the next barrier
-            if (copy) copy_out(dst((i + 1) & 1), w_q[0]);
+            if (!DROLE && copy) copy_out(dst((i + 1) & 1), w_q[0]);
             shift();
             rc = m5(rc + 1);
         };
@@ -417,7 +428,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         for (; i < n_iter; ++i) step(i, true, true, true, true);
         for (; i <= last; ++i) step(i, false, i <= n_iter, true, true);
         __syncthreads();
-        copy_out(dst((n_iter - 1) & 1), w_q[0]);
+        if (!DROLE) copy_out(dst((n_iter - 1) & 1), w_q[0]);
     };
     if (d_role) {
         if (tail_block) run(std::true_type{}, std::true_type{});
