@@ -3,6 +3,7 @@
 #include "../../include/lvx.h"
 #include "lvx_kernels.hpp"
 
+#include <algorithm>
 #include <cmath>
 
 using namespace lvx;
@@ -233,14 +234,31 @@ static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
     return (size_t)2 * s->B * s->Lkv * s->Hkv * s->D * sizeof(float);
 }
 
+// The dQ GEMM of a small row window (a one-round launch) has only B*Hq C tiles; its
+// contraction over the tokens is then split over several work-groups that add fp32
+// partial tiles into a scratch, rounded to bf16 afterwards.  Returns the number of
+// splits (1: none) and the tokens per split.
+static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_len) {
+    const int tiles = row_count > 256 ? (row_count + 511) / 512 : 1;
+    const int wgs = s->B * s->Hq * tiles;
+    const int blocks = (s->Lkv + 127) / 128;
+    int ks = 1;
+    if (wgs < 128) ks = std::min(std::min(8, 256 / wgs), blocks);
+    const int per = (blocks + ks - 1) / ks;
+    *split_len = per * 128;
+    return (blocks + per - 1) / per;
+}
+
 size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
     if (!s || row_count <= 0) return 0;
     const size_t tokens = ((size_t)s->Lkv + 127) / 128 * 128;
     const size_t rows = ((size_t)row_count + 31) / 32 * 32;
     // dS^T tiles, then fp32 dK/dV scratch for the split-steps mode with bf16 outputs, then the
     // row metadata records (2 floats per row and head)
+    int sl;
+    const size_t dq32 = dq_k_splits(s, row_count, &sl) > 1 ? (size_t)s->B * s->Hq * rows * s->D * sizeof(float) : 0;
     return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s) +
-           (size_t)s->B * s->Hq * rows * 2 * sizeof(float);
+           (size_t)s->B * s->Hq * rows * 2 * sizeof(float) + dq32;
 }
 
 int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
@@ -349,7 +367,27 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.k_len = s->kv_len;
     g.a_tiled_m = (int)(rows / 32);
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
-    return static_cast<int>(launch_gemm(g, true, true, st));
+    int split_len = 0;
+    const int ks = dq_k_splits(s, row_count, &split_len);
+    if (ks <= 1) return static_cast<int>(launch_gemm(g, true, true, st));
+    // split contraction: zero the fp32 scratch, accumulate, round into dq
+    float* dq32 = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                           (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s) +
+                                           (size_t)s->B * s->Hq * rows * 2 * sizeof(float));
+    FillParams fz{reinterpret_cast<uint32_t*>(dq32), (int64_t)s->B * s->Hq * rows * s->D * (int64_t)sizeof(float) / 16};
+    e = launch_zero(fz, st);
+    if (e != hipSuccess) return static_cast<int>(e);
+    g.k_splits = ks; g.k_split_len = split_len;
+    g.c32 = dq32; g.c32_batch = (int64_t)row_count * s->D; g.c32_ld = row_count;   // [B * Hq][D][row_count]
+    e = launch_gemm(g, true, true, st);
+    if (e != hipSuccess) return static_cast<int>(e);
+    CastParams cq{};
+    cq.src = dq32;
+    cq.dst = static_cast<uint16_t*>(dq->ptr) + (int64_t)row_begin * dq->stride_s;
+    cq.ds = st3(dq);
+    cq.B = s->B; cq.H = s->Hq; cq.L = row_count;
+    cq.transposed = 1;
+    return static_cast<int>(launch_cast(cq, st));
 }
 
 int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L, int32_t D,

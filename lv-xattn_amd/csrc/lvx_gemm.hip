@@ -109,8 +109,11 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     constexpr int NRA = RA::NRD(WM), NRB = RB::NRD(WN);
     __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
-    const int wid = xcd_remap(blockIdx.x, p.total_wg);
-    if (wid >= p.total_wg) return;
+    const int wid0 = xcd_remap(blockIdx.x, p.total_wg);
+    if (wid0 >= p.total_wg) return;
+    const int nks = p.k_splits > 1 ? p.k_splits : 1;
+    const int ksp = wid0 % nks;
+    const int wid = wid0 / nks;
     const int tn = wid % p.tiles_n;
     const int t1 = wid / p.tiles_n;
     const int tm = t1 % p.tiles_m;
@@ -124,6 +127,9 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     uint16_t* const Cz = pr.C + zo * p.c_outer + zi * p.c_inner;
     int klen0 = pr.K[0];
     if (p.k_len) klen0 = min(klen0, p.k_len[zo]);
+    const int k_lo = ksp * p.k_split_len;          // 0 without a split
+    if (nks > 1) klen0 = max(0, min(klen0, k_lo + p.k_split_len) - k_lo);
+    const int s_lo = k_lo / BK;                    // first stage of this work-group's k range
     const int klen1 = pr.nseg > 1 ? pr.K[1] : 0;
 
     const int tid = threadIdx.x;
@@ -158,8 +164,9 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
 
     auto issue = [&](int s) {     // loads of stage s into ring slot s % NS
         const int sg = s >= steps0 ? 1 : 0;
-        const int ks = sg ? s - steps0 : s;
-        const int krem = (sg ? klen1 : klen0) - ks * BK;
+        const int kr = sg ? s - steps0 : s;            // stage inside this work-group's range
+        const int krem = (sg ? klen1 : klen0) - kr * BK;
+        const int ks = sg ? kr : kr + s_lo;            // stage inside the operand
         const char* ab = abase[sg] + ks * a_kstride;
         if (A_MCONTIG && p.a_tiled_m)   // tiled A: [k / 128][m / 32][128 k][32 m]
             ab = abase[sg] + ((int64_t)(ks >> 2) * p.a_tiled_m * 4096 + (ks & 3) * (BK * 32)) * 2;
@@ -237,6 +244,26 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     if (set == 0) phase_barrier();
 
     // C^T tile: accumulator rows = n, cols = m
+    if (nks > 1) {   // partial tile of a split contraction: fp32 atomic adds
+        if (steps == 0) return;
+        float* const C32 = p.c32 + (int64_t)z * p.c32_batch;
+#pragma unroll
+        for (int mt = 0; mt < WM; ++mt) {
+            const int m = m0 + 32 * (WM * wm + mt) + l32;
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int n = n0 + 32 * (WN * wn + nt) + 8 * vg + 4 * g;
+                    if (n < p.N) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) unsafeAtomicAdd(C32 + (int64_t)(n + r) * p.c32_ld + m, acc[nt][mt][4 * vg + r]);
+                    }
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < WM; ++mt) {
         const int m = m0 + 32 * (WM * wm + mt) + l32;
@@ -261,7 +288,7 @@ hipError_t launch_cfg(GemmParams p, bool a_mcontig, bool b_ncontig, hipStream_t 
     constexpr int TM = 32 * WM * GM, TN = 32 * WN * GN;
     p.tiles_m = (p.M + TM - 1) / TM;
     p.tiles_n = (p.N + TN - 1) / TN;
-    p.total_wg = p.nprob * p.nbatch * p.tiles_m * p.tiles_n;
+    p.total_wg = p.nprob * p.nbatch * p.tiles_m * p.tiles_n * (p.k_splits > 1 ? p.k_splits : 1);
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (!a_mcontig && !b_ncontig)
         hipLaunchKernelGGL((gemm_kernel<false, false, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);

@@ -102,6 +102,7 @@ struct CastParams {
     uint16_t* dst;
     Strides3 ds;
     int B, H, L;
+    int transposed;   // 0: src is [B*H][L][D]; 1: src is [B*H][D][L]
 };
 
 // One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].
@@ -129,6 +130,15 @@ struct GemmParams {
     int nbatch, batch_inner, b_group;
     int64_t a_batch, b_outer, b_inner, c_outer, c_inner;
     const int32_t* k_len;
+    // Split contraction (single-segment problems): k_splits work-groups per C tile, each
+    // contracting k_split_len values of k (a multiple of 128) and adding its partial tile
+    // with fp32 atomics to the TRANSPOSED scratch c32[z * c32_batch + n * c32_ld + m] (zeroed
+    // by the caller; the accumulator holds C^T, so a wave's lanes then add to consecutive
+    // addresses) instead of storing bf16 to C.  k_splits <= 1: off.
+    int k_splits, k_split_len;
+    float* c32;
+    int64_t c32_batch;
+    int c32_ld;
     // a_tiled_m > 0: A (stored [K][M]) is cut into contiguous [128 k][32 m] tiles,
     // a_tiled_m of them per block of 128 k; lda is ignored
     int a_tiled_m;

@@ -147,6 +147,25 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
+// Same from a transposed source [B*H][D][L]: adjacent threads take adjacent rows, so the
+// eight strided reads of a thread are coalesced across the wave.
+__global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.B * p.H * p.L * 16) return;
+    const int row = (int)(idx % p.L);
+    const int chunk = (int)((idx / p.L) & 15);
+    const int bh = (int)(idx / ((int64_t)p.L * 16));
+    const int b = bh / p.H, h = bh % p.H;
+    const float* s = p.src + ((int64_t)bh * D + chunk * 8) * p.L + row;
+    float a[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a[j] = s[(int64_t)j * p.L];
+    u32x4 u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u[j] = pack_bf16(a[2 * j], a[2 * j + 1]);
+    *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
+}
+
 // zero fill (a kernel rather than hipMemsetAsync, so that callers may capture the stream)
 __global__ __launch_bounds__(256) void zero_kernel(const FillParams p) {
     const u32x4 z = {0u, 0u, 0u, 0u};
@@ -189,7 +208,10 @@ hipError_t launch_zero(const FillParams& p, hipStream_t st) {
 hipError_t launch_cast(const CastParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.H * p.L;
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(cast_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    if (p.transposed)
+        hipLaunchKernelGGL(cast_t_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(cast_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
