@@ -156,6 +156,32 @@ int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, in
                 int32_t M, int32_t Dm, int32_t N, void* stream);
 
 /*
+ * The same with the k_norm of `project` (`key_states = self.k_norm(key_states)`,
+ * test_llama3.py:418; MllamaTextRMSNorm of transformers 4.47.1 over head_dim)
+ * applied to K in the GEMM's epilogue, per row and per head of 128 columns:
+ *   x = bf16(X W_k),  r = rsqrt(mean_d(x^2) + eps),  K = bf16(w * bf16(x * r)).
+ * N must be a multiple of 128.  k_norm_w: 128 bf16 weights, 16-byte aligned.
+ * Optional outputs for the norm's backward (null: not written):
+ *   k_raw  : x, indexed like k_out (row stride ldkv);
+ *   k_rstd : r, fp32 [M, N / 128].
+ */
+int lvx_kv_proj_norm(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw,
+                     int32_t w_in_major, void* k_out, void* v_out, int64_t ldkv,
+                     int32_t M, int32_t Dm, int32_t N, const void* k_norm_w, float eps,
+                     void* k_raw, float* k_rstd, void* stream);
+
+/*
+ * Backward of that norm (what autograd derives for test_llama3.py:418 when the
+ * K/V gradients are propagated, which the reference's wrapper does not do,
+ * :243): with xh = k_raw * r and g = dk * w, per row and head
+ *   dk_raw = r * (g - xh * mean_d(g * xh)),   dw[d] += sum over rows, heads of dk * bf16(xh).
+ * dk_raw may alias dk.  dw: fp32 [128], ADDED to (null: not wanted).
+ */
+int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk, const float* k_rstd,
+                   const void* k_norm_w, void* dk_raw, int64_t lddk_raw, float* dw,
+                   int32_t M, int32_t N, void* stream);
+
+/*
  * dX[M, Dm] = dK[M, N] * W_k^T + dV[M, N] * W_v^T  (no counterpart in the
  * reference, whose wrapper drops this gradient: test_llama3.py:243).
  */

@@ -424,8 +424,9 @@ static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch = 1) {
 
 extern "C" {
 
-int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
-                void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, void* stream) {
+static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
+                        void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N,
+                        const void* k_norm_w, float eps, void* k_raw, float* k_rstd, void* stream) {
     LVX_TRY(check_gemm_ptr(x, ldx));
     LVX_TRY(check_gemm_ptr(w_k, ldw));
     LVX_TRY(check_gemm_ptr(w_v, ldw));
@@ -443,8 +444,57 @@ int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, in
         pr.K[0] = Dm; pr.nseg = 1;
         pr.C = static_cast<uint16_t*>(c[i]); pr.ldc = ldkv;
     }
+    if (k_norm_w) {
+        if (N % 128) return LVX_ERR_HEAD_DIM;      // the norm runs over heads of 128 columns
+        if (!aligned16(k_norm_w)) return LVX_ERR_ALIGN;
+        if (!(eps >= 0.f)) return LVX_ERR_SHAPE;
+        if (k_raw) LVX_TRY(check_gemm_ptr(k_raw, ldkv));
+        if (k_rstd && (reinterpret_cast<uintptr_t>(k_rstd) & 3)) return LVX_ERR_ALIGN;
+        g.norm_w = static_cast<const uint16_t*>(k_norm_w);
+        g.norm_eps = eps;
+        g.c_raw = static_cast<uint16_t*>(k_raw);
+        g.rstd = k_rstd;
+    }
     fill_grid(g, M, N, 2);
     return static_cast<int>(launch_gemm(g, false, w_in_major != 0, static_cast<hipStream_t>(stream)));
+}
+
+int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
+                void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, void* stream) {
+    return kv_proj_impl(x, ldx, w_k, w_v, ldw, w_in_major, k_out, v_out, ldkv, M, Dm, N, nullptr, 0.f, nullptr,
+                        nullptr, stream);
+}
+
+int lvx_kv_proj_norm(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
+                     void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N,
+                     const void* k_norm_w, float eps, void* k_raw, float* k_rstd, void* stream) {
+    if (!k_norm_w) return LVX_ERR_NULL;
+    return kv_proj_impl(x, ldx, w_k, w_v, ldw, w_in_major, k_out, v_out, ldkv, M, Dm, N, k_norm_w, eps, k_raw,
+                        k_rstd, stream);
+}
+
+int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk, const float* k_rstd,
+                   const void* k_norm_w, void* dk_raw, int64_t lddk_raw, float* dw, int32_t M, int32_t N,
+                   void* stream) {
+    LVX_TRY(check_gemm_ptr(dk, lddk));
+    LVX_TRY(check_gemm_ptr(k_raw, ldk));
+    LVX_TRY(check_gemm_ptr(dk_raw, lddk_raw));
+    if (!k_rstd || !k_norm_w) return LVX_ERR_NULL;
+    if (!aligned16(k_norm_w) || (reinterpret_cast<uintptr_t>(k_rstd) & 3) || (reinterpret_cast<uintptr_t>(dw) & 3))
+        return LVX_ERR_ALIGN;
+    if (M <= 0 || N <= 0) return LVX_ERR_SHAPE;
+    if (N % 128) return LVX_ERR_HEAD_DIM;
+    if (lddk < N || ldk < N || lddk_raw < N) return LVX_ERR_SHAPE;
+    NormBwdParams p{};
+    p.dy = static_cast<const uint16_t*>(dk);
+    p.x = static_cast<const uint16_t*>(k_raw);
+    p.rstd = k_rstd;
+    p.w = static_cast<const uint16_t*>(k_norm_w);
+    p.dx = static_cast<uint16_t*>(dk_raw);
+    p.dw = dw;
+    p.ldy = lddk; p.ldx = ldk; p.lddx = lddk_raw;
+    p.M = M; p.heads = N / 128;
+    return static_cast<int>(launch_norm_bwd(p, static_cast<hipStream_t>(stream)));
 }
 
 int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v, int64_t ldw,

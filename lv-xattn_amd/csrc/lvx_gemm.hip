@@ -264,6 +264,67 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
         }
         return;
     }
+    if (p.norm_w && t2 / p.nbatch == 0) {
+        // RMS norm over each 128-column group (N and the tile are multiples of 128): the
+        // group's columns sit in HW = 4 / WN waves with consecutive wn; row sums of squares
+        // are exchanged through LDS, which no wave reads any more.
+        constexpr int HW = 4 / WN;
+        static_assert(WN == 2 || WN == 4, "a 128-column group spans 1 or 2 waves");
+        float* const red = reinterpret_cast<float*>(lds);
+        float rs[WM];
+#pragma unroll
+        for (int mt = 0; mt < WM; ++mt) {
+            float ss = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float x = bf16_hi(pack_bf16(0.f, acc[nt][mt][i]));   // the product as bf16
+                    acc[nt][mt][i] = x;
+                    ss = fmaf(x, x, ss);
+                }
+            ss += __shfl_xor(ss, 32);
+            rs[mt] = ss;
+            if (HW > 1 && g == 0) red[(wave * WM + mt) * 32 + l32] = ss;
+        }
+        if (HW > 1) {
+            __syncthreads();
+            const int pw = wm + GM * (wn ^ 1);
+#pragma unroll
+            for (int mt = 0; mt < WM; ++mt) rs[mt] += red[(pw * WM + mt) * 32 + l32];
+        }
+        const int groups = p.N >> 7;
+#pragma unroll
+        for (int mt = 0; mt < WM; ++mt) {
+            const int m = m0 + 32 * (WM * wm + mt) + l32;
+            if (m >= p.M) continue;
+            const float r = rsqrtf(rs[mt] * (1.f / 128.f) + p.norm_eps);
+            const int ncol = n0 + 32 * WN * wn;
+            if (p.rstd && g == 0 && (wn & (HW - 1)) == 0 && ncol < p.N) p.rstd[(int64_t)m * groups + (ncol >> 7)] = r;
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int n = n0 + 32 * (WN * wn + nt) + 8 * vg + 4 * g;
+                    if (n < p.N) {
+                        const float a[4] = {acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1], acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]};
+                        if (p.c_raw) {
+                            u32x2 w;
+                            w[0] = pack_bf16(a[0], a[1]);
+                            w[1] = pack_bf16(a[2], a[3]);
+                            *reinterpret_cast<u32x2*>(p.c_raw + (Cz - pr.C) + (int64_t)m * pr.ldc + n) = w;
+                        }
+                        const u32x2 wt = *reinterpret_cast<const u32x2*>(p.norm_w + (n & 127));
+                        const u32x2 h = {pack_bf16(a[0] * r, a[1] * r), pack_bf16(a[2] * r, a[3] * r)};
+                        u32x2 y;
+                        y[0] = pack_bf16(bf16_lo(wt[0]) * bf16_lo(h[0]), bf16_hi(wt[0]) * bf16_hi(h[0]));
+                        y[1] = pack_bf16(bf16_lo(wt[1]) * bf16_lo(h[1]), bf16_hi(wt[1]) * bf16_hi(h[1]));
+                        *reinterpret_cast<u32x2*>(Cz + (int64_t)m * pr.ldc + n) = y;
+                    }
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < WM; ++mt) {
         const int m = m0 + 32 * (WM * wm + mt) + l32;

@@ -130,6 +130,15 @@ struct GemmParams {
     int nbatch, batch_inner, b_group;
     int64_t a_batch, b_outer, b_inner, c_outer, c_inner;
     const int32_t* k_len;
+    // RMS norm over each aligned group of 128 columns of problem 0's C (the k_norm of the K
+    // projection), applied to the accumulator before the store: y = bf16(w * bf16(x * r)),
+    // r = rsqrt(mean(x^2) + eps), x = the bf16-rounded product.  norm_w: 128 bf16 weights
+    // (null: off).  c_raw (optional): x itself, indexed like C.  rstd (optional):
+    // r[m * (N / 128) + n / 128].
+    const uint16_t* norm_w;
+    float norm_eps;
+    uint16_t* c_raw;
+    float* rstd;
     // Split contraction (single-segment problems): k_splits work-groups per C tile, each
     // contracting k_split_len values of k (a multiple of 128) and adding its partial tile
     // with fp32 atomics to the TRANSPOSED scratch c32[z * c32_batch + n * c32_ld + m] (zeroed
@@ -151,6 +160,19 @@ hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);
 hipError_t launch_cast(const CastParams& p, hipStream_t st);
 hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st);
 hipError_t launch_zero(const FillParams& p, hipStream_t st);
+
+// Backward of the 128-wide RMS norm: rows of dy, x [M][heads][128] (row strides ldy, ldx), r [M][heads].
+struct NormBwdParams {
+    const uint16_t* dy;
+    const uint16_t* x;
+    const float* rstd;
+    const uint16_t* w;
+    uint16_t* dx;
+    float* dw;        // [128] fp32, added to (null: not wanted)
+    int64_t ldy, ldx, lddx;
+    int M, heads;
+};
+hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st);
 // a_mcontig: A is stored [K][M] (m contiguous); b_ncontig: B is stored [K][N].
 hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st);
 

@@ -6,6 +6,8 @@
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
+#include <algorithm>
+
 namespace lvx {
 
 namespace {
@@ -166,6 +168,62 @@ __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
+// Backward of y = w * bf16(x * r) over 128-wide rows: with xh = x * r and gg = dy * w,
+//   dx = r * (gg - xh * mean(gg * xh)),   dw += sum over rows of dy * bf16(xh).
+// 16 lanes per row (8 columns each); a thread keeps the dw partial sums of its 8 columns
+// over the rows it visits, the block folds them through LDS and adds them with atomics.
+__global__ __launch_bounds__(256) void norm_bwd_kernel(const NormBwdParams p) {
+    __shared__ float fold[16][16][8];
+    const int sub = threadIdx.x & 15, grp = threadIdx.x >> 4;
+    const int64_t nrows = (int64_t)p.M * p.heads;
+    const u32x4 wu = *reinterpret_cast<const u32x4*>(p.w + sub * 8);
+    float w[8], dwp[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { w[2 * j] = bf16_lo(wu[j]); w[2 * j + 1] = bf16_hi(wu[j]); }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dwp[j] = 0.f;
+    for (int64_t row = (int64_t)blockIdx.x * 16 + grp; row < nrows; row += (int64_t)gridDim.x * 16) {
+        const int64_t m = row / p.heads;
+        const int h = (int)(row % p.heads);
+        const u32x4 du = *reinterpret_cast<const u32x4*>(p.dy + m * p.ldy + h * 128 + sub * 8);
+        const u32x4 xu = *reinterpret_cast<const u32x4*>(p.x + m * p.ldx + h * 128 + sub * 8);
+        const float r = p.rstd[row];
+        float gg[8], xh[8], c = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float d0 = bf16_lo(du[j]), d1 = bf16_hi(du[j]);
+            xh[2 * j] = bf16_lo(xu[j]) * r;
+            xh[2 * j + 1] = bf16_hi(xu[j]) * r;
+            gg[2 * j] = d0 * w[2 * j];
+            gg[2 * j + 1] = d1 * w[2 * j + 1];
+            const uint32_t xb = pack_bf16(xh[2 * j], xh[2 * j + 1]);
+            dwp[2 * j] = fmaf(d0, bf16_lo(xb), dwp[2 * j]);
+            dwp[2 * j + 1] = fmaf(d1, bf16_hi(xb), dwp[2 * j + 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c = fmaf(gg[j], xh[j], c);
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) c += __shfl_xor(c, o);
+        c *= 1.f / 128.f;
+        u32x4 out;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            out[j] = pack_bf16(r * (gg[2 * j] - xh[2 * j] * c), r * (gg[2 * j + 1] - xh[2 * j + 1] * c));
+        *reinterpret_cast<u32x4*>(p.dx + m * p.lddx + h * 128 + sub * 8) = out;
+    }
+    if (!p.dw) return;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fold[grp][sub][j] = dwp[j];
+    __syncthreads();
+    if (threadIdx.x < 128) {
+        const int s2 = threadIdx.x >> 3, j = threadIdx.x & 7;
+        float t = 0.f;
+#pragma unroll
+        for (int gi = 0; gi < 16; ++gi) t += fold[gi][s2][j];
+        unsafeAtomicAdd(p.dw + threadIdx.x, t);
+    }
+}
+
 // zero fill (a kernel rather than hipMemsetAsync, so that callers may capture the stream)
 __global__ __launch_bounds__(256) void zero_kernel(const FillParams p) {
     const u32x4 z = {0u, 0u, 0u, 0u};
@@ -202,6 +260,14 @@ hipError_t launch_zero(const FillParams& p, hipStream_t st) {
     if (p.n16 <= 0) return hipSuccess;
     const int grid = (int)((p.n16 + 255) / 256 < 4096 ? (p.n16 + 255) / 256 : 4096);
     hipLaunchKernelGGL(zero_kernel, dim3(grid), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.M * p.heads;
+    if (rows == 0) return hipSuccess;
+    const int grid = (int)std::min<int64_t>((rows + 15) / 16, 2048);
+    hipLaunchKernelGGL(norm_bwd_kernel, dim3(grid), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 

@@ -51,6 +51,10 @@ SYMBOLS = {
     "lvx_cast_f32_bf16": (C.c_int, [_P, _T, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_kv_proj": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, _P, C.c_int64,
                               C.c_int32, C.c_int32, C.c_int32, _P]),
+    "lvx_kv_proj_norm": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, _P, C.c_int64,
+                                   C.c_int32, C.c_int32, C.c_int32, _P, C.c_float, _P, _P, _P]),
+    "lvx_k_norm_bwd": (C.c_int, [_P, C.c_int64, _P, C.c_int64, _P, _P, _P, C.c_int64, _P,
+                                 C.c_int32, C.c_int32, _P]),
     "lvx_dx_vis": (C.c_int, [_P, _P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, C.c_int64,
                              C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_dw_kv": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, _P, _P, C.c_int64, C.c_int32,

@@ -69,37 +69,60 @@ class KVProjection:
 
 def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = False,
                            rounds: Optional[int] = None, batched: bool = False,
-                           weight_grads: bool = False):
-    """apply(q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None) -> o
+                           weight_grads: bool = False, w_in_major: bool = True):
+    """apply(q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None, k_norm_weight=None,
+    k_norm_eps=1e-5, bias_func=None, *bias_args) -> o
 
     Forward: K, V = kv_proj(x_vis); o, L = attention; saves (q, x_vis, w_k, w_v,
     o, L) - K and V are dropped.  Backward: recomputes K, V by the same GEMMs,
     runs the attention backward, then dX_vis = dK W_k^T + dV W_v^T (and, with
-    `weight_grads`, dW_k = X^T dK, dW_v = X^T dV)."""
+    `weight_grads`, dW_k = X^T dK, dW_v = X^T dV).  With `k_norm_weight` K is
+    RMS-normalised per head in the projection's epilogue (the k_norm of
+    test_llama3.py:418) and backward goes through the norm before dX_vis
+    (weight_grads: also returns the norm weight's gradient).  `w_in_major`:
+    W is [Dm, Hkv*D]; False: [Hkv*D, Dm] (torch.nn.Linear.weight).
+    `bias_func(*bias_args)` gives the dense additive bias, as for
+    `_attn_forward`; the arguments are kept and the bias is rebuilt in backward."""
     if attention_mode != "lv_xattn":
         raise ValueError("only attention_mode='lv_xattn' exists on this path")
 
     class _attention(torch.autograd.Function):
         @staticmethod
-        def forward(ctx, q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None):
-            k, v = ops.kv_proj(x_vis, w_k, w_v, n_kv_heads)
-            _, _, _, o, L = _attn_forward(q, k, v, False, sm_scale, None, no_overlap=no_overlap,
-                                          rounds=rounds, mask=mask, batched=batched)
-            ctx.save_for_backward(q, x_vis, w_k, w_v, o, L)
+        def forward(ctx, q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None, k_norm_weight=None,
+                    k_norm_eps=1e-5, bias_func=None, *bias_args):
+            k, v = ops.kv_proj(x_vis, w_k, w_v, n_kv_heads, w_in_major, k_norm_weight=k_norm_weight,
+                               eps=k_norm_eps)
+            _, _, _, o, L = _attn_forward(q, k, v, False, sm_scale, None, bias_func, list(bias_args), [],
+                                          no_overlap, rounds=rounds, mask=mask, batched=batched)
+            ctx.has_norm = k_norm_weight is not None
+            ctx.save_for_backward(q, x_vis, w_k, w_v, o, L, *([k_norm_weight] if ctx.has_norm else []), *bias_args)
+            ctx.k_norm_eps, ctx.bias_func, ctx.n_bias = k_norm_eps, bias_func, len(bias_args)
             ctx.n_kv_heads, ctx.sm_scale, ctx.mask = n_kv_heads, sm_scale, mask
             reset_global_memory_buffer(attention_mode)
             return o
 
         @staticmethod
         def backward(ctx, do):
-            q, x_vis, w_k, w_v, o, L = ctx.saved_tensors
-            k, v = ops.kv_proj(x_vis, w_k, w_v, ctx.n_kv_heads)          # recompute
+            q, x_vis, w_k, w_v, o, L, *rest = ctx.saved_tensors
+            norm_w = rest[0] if ctx.has_norm else None
+            bias_args = rest[1:] if ctx.has_norm else rest
+            dwn = None
+            if ctx.has_norm:                                             # recompute, keeping x and r
+                k, v, k_raw, k_rstd = ops.kv_proj(x_vis, w_k, w_v, ctx.n_kv_heads, w_in_major,
+                                                  k_norm_weight=norm_w, eps=ctx.k_norm_eps, for_backward=True)
+            else:
+                k, v = ops.kv_proj(x_vis, w_k, w_v, ctx.n_kv_heads, w_in_major)
             dq, dk, dv = _attn_backward(do, q, k, v, o, L, False, ctx.sm_scale, None, "flash",
-                                        no_overlap=no_overlap, rounds=rounds, mask=ctx.mask, batched=batched)
-            dx = ops.dx_vis(dk, dv, w_k, w_v)
+                                        ctx.bias_func, list(bias_args), [], no_overlap,
+                                        rounds=rounds, mask=ctx.mask, batched=batched)
+            if ctx.has_norm:
+                dk, dwn = ops.k_norm_bwd(dk, k_raw, k_rstd, norm_w, want_dw=weight_grads)
+                if dwn is not None:
+                    dwn = dwn.to(norm_w.dtype)
+            dx = ops.dx_vis(dk, dv, w_k, w_v, w_in_major)
             dwk = dwv = None
             if weight_grads:
-                dwk, dwv = ops.dw_kv(x_vis, dk, dv)
-            return dq, dx, dwk, dwv, None, None, None
+                dwk, dwv = ops.dw_kv(x_vis, dk, dv, w_in_major)
+            return (dq, dx, dwk, dwv, None, None, None, dwn, None, None) + (None,) * ctx.n_bias
 
     return _attention

@@ -14,8 +14,17 @@ Q [B,Hq,Lq,D], K, V [B,Hkv,Lkv,D] and the additive cross-attention mask
 [B,1,Lq,Lkv] to `lv_xattn_attention_forward`, which runs the gfx950 flash
 forward / backward (dense-bias variant; K/V kept for backward, as in the
 reference's `create_attention_class_save_qkv`, test_llama3.py:125-178).
-Self-attention layers and anything the kernels do not cover (head_dim other
-than 128, dropout, a causal request) fall back to transformers' eager path.
+The registry is model-wide, so the causal self-attention layers arrive here as
+well; they are not this operator and are passed on to transformers' own
+implementation.  A cross-attention call the kernels do not cover (not bf16 on
+the GPU, head_dim other than 128, dropout) raises.
+
+`patch_cross_attention_forward(model)` goes one step further, like the
+reference's recompute variant (`create_attention_class`,
+test_llama3.py:180-245, used by the patched forward at :361-466): the K/V
+projections and the k_norm move inside the autograd function, so K and V are
+not kept between forward and backward but recomputed from the visual hidden
+states by the gfx950 GEMM (norm fused in its epilogue).
 """
 from __future__ import annotations
 
@@ -23,7 +32,8 @@ from typing import Optional
 
 import torch
 
-from .autograd import create_attention_class_save_qkv
+from ._lib import LvxError
+from .autograd import create_attention_class, create_attention_class_save_qkv
 
 NAME = "lv_xattn"
 _attention = None
@@ -47,13 +57,12 @@ def lv_xattn_attention_forward(module, query, key, value, attention_mask: Option
     """Attention-interface function (same contract as transformers'
     eager_attention_forward): returns (attn_output [B, Lq, Hq, D], None)."""
     global _attention
-    usable = (query.is_cuda and query.dtype == torch.bfloat16 and query.shape[-1] == 128 and dropout == 0.0
-              and not kwargs.get("is_causal", False) and getattr(module, "is_causal", False) is not True
-              and query.shape[1] % key.shape[1] == 0)
-    if not usable:
+    if kwargs.get("is_causal", False) or getattr(module, "is_causal", False) is True or not hasattr(module, "k_norm"):
+        # a (causal) self-attention layer: another operator, transformers' own
         from transformers.models.mllama.modeling_mllama import eager_attention_forward
         return eager_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
                                        scaling=scaling, **kwargs)
+    _require_supported(query, key, dropout)
     if _attention is None:
         _attention = create_attention_class_save_qkv("lv_xattn", rounds=1, batched=True).apply
     if scaling is None:
@@ -65,6 +74,67 @@ def lv_xattn_attention_forward(module, query, key, value, attention_mask: Option
         mask = attention_mask[..., :Lq, :Lkv]
         out = _attention(query, key, value, False, scaling, _mask_bias, [mask], [])
     return out.transpose(1, 2).contiguous(), None
+
+
+def _require_supported(query, key, dropout):
+    if not (query.is_cuda and query.dtype == torch.bfloat16 and query.shape[-1] == 128 and dropout == 0.0
+            and query.shape[1] % key.shape[1] == 0):
+        raise LvxError("lv_xattn cross-attention needs bf16 tensors on the GPU, head_dim 128, no dropout and "
+                       f"Hkv | Hq; got {query.dtype} on {query.device}, q {tuple(query.shape)}, "
+                       f"k {tuple(key.shape)}, dropout {dropout}")
+
+
+_recompute = {}
+
+
+def _recompute_forward(self, hidden_states, cross_attention_states=None, past_key_values=None,
+                       attention_mask=None, use_cache=None, **kwargs):
+    """Replacement for MllamaTextCrossAttention.forward with the K/V recompute
+    of the reference's patched forward (test_llama3.py:361-466).  Extra
+    keyword `lvx_mask`: a compact `Mask` (see mask_from_cross_attention_mask)
+    used instead of the dense `attention_mask`."""
+    if cross_attention_states is None or past_key_values is not None:
+        # decoding from a K/V cache: nothing to recompute; the stock forward
+        # still reaches the kernels through the attention interface
+        return self._lvx_stock_forward(hidden_states, cross_attention_states, past_key_values,
+                                       attention_mask, use_cache, **kwargs)
+    bsz, q_len, _ = hidden_states.size()
+    query = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+    query = self.q_norm(query)
+    dropout = self.dropout if self.training else 0.0
+    if not (query.is_cuda and query.dtype == torch.bfloat16 and self.head_dim == 128 and dropout == 0.0):
+        raise LvxError("lv_xattn cross-attention needs bf16 tensors on the GPU, head_dim 128 and no dropout")
+    key = (self._lvx_rounds, self._lvx_batched, self._lvx_weight_grads)
+    if key not in _recompute:
+        _recompute[key] = create_attention_class("lv_xattn", rounds=key[0], batched=key[1],
+                                                 weight_grads=key[2], w_in_major=False).apply
+    mask = kwargs.get("lvx_mask")
+    bias = []
+    if mask is None and attention_mask is not None:
+        lkv = cross_attention_states.shape[1]
+        bias = [_mask_bias, attention_mask[..., :q_len, :lkv]]
+    out = _recompute[key](query, cross_attention_states.to(query.dtype), self.k_proj.weight, self.v_proj.weight,
+                          self.num_key_value_heads, self.scaling, mask, self.k_norm.weight,
+                          self.k_norm.variance_epsilon, *bias)
+    out = out.transpose(1, 2).reshape(bsz, q_len, -1)
+    return self.o_proj(out), None
+
+
+def patch_cross_attention_forward(model, rounds: int = 1, batched: bool = True, weight_grads: bool = True) -> int:
+    """Installs the recompute forward on every MllamaTextCrossAttention module
+    under `model` (the reference assigns its patched forward to the class,
+    test_llama3.py:666-668; here it is per instance, so unpatching is
+    `del module.forward`).  Returns the number of modules patched."""
+    import types
+    from transformers.models.mllama.modeling_mllama import MllamaTextCrossAttention
+    n = 0
+    for mod in model.modules():
+        if isinstance(mod, MllamaTextCrossAttention):
+            mod._lvx_stock_forward = types.MethodType(MllamaTextCrossAttention.forward, mod)
+            mod._lvx_rounds, mod._lvx_batched, mod._lvx_weight_grads = rounds, batched, weight_grads
+            mod.forward = types.MethodType(_recompute_forward, mod)
+            n += 1
+    return n
 
 
 def register() -> str:

@@ -158,10 +158,16 @@ def _rows2d(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
     return t2.data_ptr(), t2.shape[0], t2.stride(0)
 
 
-def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True):
+def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True,
+            k_norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5, for_backward: bool = False):
     """K, V = X W_k, X W_v.  x_vis [B, Lkv, Dm]; W [Dm, Hkv*D] (w_in_major) or
     [Hkv*D, Dm] (torch.nn.Linear.weight).  Returns [B, Hkv, Lkv, D] views of
-    [B, Lkv, Hkv, D] memory."""
+    [B, Lkv, Hkv, D] memory.
+
+    With `k_norm_weight` ([D] bf16) K is RMS-normalised per head in the GEMM's
+    epilogue (the k_norm of test_llama3.py:418 in the reference).  With
+    `for_backward` the call also returns what the norm's backward needs:
+    (k, v, k_raw [B,Hkv,Lkv,D] view, k_rstd fp32 [B, Lkv, Hkv])."""
     B, Lkv, Dm = x_vis.shape
     N = w_k.shape[1] if w_in_major else w_k.shape[0]
     xp, M, ldx = _rows2d(x_vis, "x_vis")
@@ -169,13 +175,60 @@ def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True):
     wvp, _, ldw2 = _rows2d(w_v, "w_v")
     if ldw != ldw2 or w_k.shape != w_v.shape:
         raise LvxError("w_k and w_v must have the same shape")
+    D = N // n_kv_heads
     k = torch.empty(B, Lkv, N, dtype=torch.bfloat16, device=x_vis.device)
     v = torch.empty_like(k)
-    rc = load().lvx_kv_proj(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
-                            M, Dm, N, stream_ptr())
-    check(rc, "lvx_kv_proj")
-    D = N // n_kv_heads
-    return (k.view(B, Lkv, n_kv_heads, D).transpose(1, 2), v.view(B, Lkv, n_kv_heads, D).transpose(1, 2))
+
+    def heads(t):
+        return t.view(B, Lkv, n_kv_heads, D).transpose(1, 2)
+
+    if k_norm_weight is None:
+        if for_backward:
+            raise LvxError("for_backward only applies with k_norm_weight")
+        rc = load().lvx_kv_proj(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
+                                M, Dm, N, stream_ptr())
+        check(rc, "lvx_kv_proj")
+        return heads(k), heads(v)
+    wn = _norm_weight(k_norm_weight, D, x_vis.device)
+    k_raw = torch.empty_like(k) if for_backward else None
+    rstd = torch.empty(B, Lkv, n_kv_heads, dtype=torch.float32, device=x_vis.device) if for_backward else None
+    rc = load().lvx_kv_proj_norm(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
+                                 M, Dm, N, wn.data_ptr(), float(eps),
+                                 k_raw.data_ptr() if for_backward else None,
+                                 rstd.data_ptr() if for_backward else None, stream_ptr())
+    check(rc, "lvx_kv_proj_norm")
+    if for_backward:
+        return heads(k), heads(v), heads(k_raw), rstd
+    return heads(k), heads(v)
+
+
+def _norm_weight(w: torch.Tensor, D: int, dev) -> torch.Tensor:
+    if w.dtype != torch.bfloat16 or tuple(w.shape) != (D,) or D != 128:
+        raise LvxError(f"k_norm_weight must be bf16 [128], got {w.dtype} {tuple(w.shape)}")
+    w = w.detach()
+    if w.device != dev:
+        raise LvxError("k_norm_weight is on another device")
+    if not w.is_contiguous() or w.data_ptr() % 16:
+        w = w.contiguous().clone()
+    return w
+
+
+def k_norm_bwd(dk, k_raw, k_rstd, k_norm_weight, want_dw: bool = True):
+    """Backward of the fused k_norm: returns (dk_raw, dw) with dk_raw a
+    [B,Hkv,Lkv,D] view of new [B,Lkv,Hkv,D] memory and dw fp32 [D] (None
+    unless `want_dw`)."""
+    B, Hkv, Lkv, D = dk.shape
+    dk2, kr2 = _token_major(dk, "dk"), _token_major(k_raw, "k_raw")
+    N = Hkv * D
+    wn = _norm_weight(k_norm_weight, D, dk.device)
+    if k_rstd.dtype != torch.float32 or k_rstd.numel() != B * Lkv * Hkv or not k_rstd.is_contiguous():
+        raise LvxError("k_rstd must be contiguous fp32 [B, Lkv, Hkv]")
+    out = torch.empty(B, Lkv, N, dtype=torch.bfloat16, device=dk.device)
+    dw = torch.zeros(D, dtype=torch.float32, device=dk.device) if want_dw else None
+    rc = load().lvx_k_norm_bwd(dk2.data_ptr(), N, kr2.data_ptr(), N, k_rstd.data_ptr(), wn.data_ptr(),
+                               out.data_ptr(), N, dw.data_ptr() if want_dw else None, B * Lkv, N, stream_ptr())
+    check(rc, "lvx_k_norm_bwd")
+    return out.view(B, Lkv, Hkv, D).transpose(1, 2), dw
 
 
 def _token_major(t: torch.Tensor, name: str) -> torch.Tensor:

@@ -27,6 +27,12 @@ by ``tests/test_oracle_*.py``:
 * ``kv_project`` / ``dx_vis`` - the K/V projections of test_llama3.py:395-398
   (two GEMMs) and their input gradient (closed form; the reference drops this
   gradient, test_llama3.py:243).  Pinned against autograd.
+* ``k_rms_norm`` / ``k_rms_norm_backward`` - the k_norm of test_llama3.py:418:
+  MllamaTextRMSNorm of transformers 4.47.1 (requirements.txt:68; a dependency,
+  absent from the reference checkout), whose published algorithm is
+  w * (x * rsqrt(mean(x^2) + eps)) with the statistics in fp32.  Pinned against
+  the MllamaTextRMSNorm class of the installed transformers, a hand-computed
+  case, and (backward) autograd and float64 finite differences.
 
 Reference quirks deliberately NOT restated (all are bugs or sit inside the
 stated tolerance): the travelling LSE initialised to 0 instead of -inf
@@ -250,6 +256,26 @@ def dw_kv(x_vis, dk, dv):
     return torch.matmul(x2.t(), dk2), torch.matmul(x2.t(), dv2)
 
 
+def k_rms_norm(k, weight, eps: float = 1e-5):
+    """y = w * x * rsqrt(mean_d(x^2) + eps) over the last (head) dimension:
+    `key_states = self.k_norm(key_states)`, test_llama3.py:418."""
+    x = k.float()
+    r = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return weight.float() * (x * r)
+
+
+def k_rms_norm_backward(dy, k_raw, weight, eps: float = 1e-5):
+    """(dx, dw) of k_rms_norm in closed form: with xh = x r and g = dy w,
+    dx = r (g - xh mean_d(g xh)), dw = sum over all rows of dy xh."""
+    x, dy, w = k_raw.float(), dy.float(), weight.float()
+    r = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    xh = x * r
+    g = dy * w
+    dx = r * (g - xh * (g * xh).mean(-1, keepdim=True))
+    dw = (dy * xh).reshape(-1, x.shape[-1]).sum(0)
+    return dx, dw
+
+
 # --------------------------------------------------------------------------
 # workloads (the five configurations the build is measured and checked on)
 # --------------------------------------------------------------------------
@@ -368,16 +394,21 @@ def n_pairs(w: Workload) -> int:
     return w.B * w.Lq * w.Lkv
 
 
-def layer_reference(w: Workload, backward: bool = True, rounds_bwd: Optional[int] = None):
-    """One cross-attention layer on the oracle: (K/V projection,) round-loop
-    forward, and optionally backward incl. dX_vis.  Returns a dict of fp32
-    tensors.  K/V are rounded to the workload dtype after the projection, as
-    the device path stores them."""
+def layer_reference(w: Workload, backward: bool = True, rounds_bwd: Optional[int] = None,
+                    k_norm_weight=None, k_norm_eps: float = 1e-5):
+    """One cross-attention layer on the oracle: (K/V projection (+ k_norm),)
+    round-loop forward, and optionally backward incl. dX_vis.  Returns a dict
+    of fp32 tensors.  K/V are rounded to the workload dtype after the
+    projection, as the device path stores them."""
     t = w.tensors
     out = {}
+    k_raw = None
     if w.Dm > 0:
         k, v = kv_project(t["x_vis"], t["w_k"], t["w_v"], w.Hkv)
         k, v = k.to(w.dtype), v.to(w.dtype)
+        if k_norm_weight is not None:
+            k_raw = k
+            k = k_rms_norm(k_raw, k_norm_weight, k_norm_eps).to(w.dtype)
         out["k"], out["v"] = k.float(), v.float()
     else:
         k, v = t["k"], t["v"]
@@ -390,5 +421,8 @@ def layer_reference(w: Workload, backward: bool = True, rounds_bwd: Optional[int
                                         allowed=allowed, rounds=rounds_bwd or w.rounds)
         out["dq"], out["dk"], out["dv"] = dq, dk, dv
         if w.Dm > 0:
+            if k_raw is not None:
+                dk, out["dw_norm"] = k_rms_norm_backward(dk.to(w.dtype), k_raw, k_norm_weight, k_norm_eps)
+                out["dk_raw"] = dk
             out["dx_vis"] = dx_vis(dk.to(w.dtype), dv.to(w.dtype), t["w_k"], t["w_v"])
     return out

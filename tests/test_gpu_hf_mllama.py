@@ -19,10 +19,17 @@ def _layer(impl):
     cfg._attn_implementation = impl
     torch.manual_seed(3)
     layer = m.MllamaTextCrossAttention(cfg, layer_idx=1)
+    with torch.no_grad():          # norm weights other than the all-ones initialisation
+        layer.q_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
+        layer.k_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
     return layer.to(device=DEV, dtype=torch.bfloat16)
 
 
-def test_mllama_cross_attention_layer_matches_eager():
+@pytest.mark.parametrize("variant", ["interface", "recompute", "recompute_intervals"])
+def test_mllama_cross_attention_layer_matches_eager(variant):
+    """interface: the attention-interface hook (K/V kept for backward);
+    recompute: the patched forward (K/V + k_norm recomputed by the fused GEMM),
+    with the dense mask or with the same mask as per-row key intervals."""
     pytest.importorskip("transformers")
     import lv_xattn
     from lv_xattn import _lib, hf_mllama
@@ -31,6 +38,8 @@ def test_mllama_cross_attention_layer_matches_eager():
     ref, new = _layer("eager"), _layer(name)
     new.load_state_dict(ref.state_dict())
     assert ref.head_dim == 128
+    if variant != "interface":
+        assert hf_mllama.patch_cross_attention_forward(new) == 1
 
     g = torch.Generator().manual_seed(11)
     B, Lq, Lkv = 2, 200, 1601
@@ -51,10 +60,18 @@ def test_mllama_cross_attention_layer_matches_eager():
     live = (mask[:, 0] > neg / 2).any(-1)                  # [B, Lq]
     go = go * live[..., None]
 
+    extra = {}
+    if variant == "recompute_intervals":
+        start = torch.zeros(B, Lq, dtype=torch.int32)
+        end = torch.full((B, Lq), Lkv, dtype=torch.int32)
+        end[0, :17] = 0
+        end[1, :] = 800
+        extra["lvx_mask"] = lv_xattn.Mask(None, start.to(DEV), end.to(DEV))
+
     outs = []
     for layer in (ref, new):
         xi, vi = x.clone().requires_grad_(), vis.clone().requires_grad_()
-        o, _ = layer(xi, cross_attention_states=vi, attention_mask=mask)
+        o, _ = layer(xi, cross_attention_states=vi, attention_mask=mask, **(extra if layer is new else {}))
         o.backward(go)
         torch.cuda.synchronize()
         outs.append((o.detach().float(), xi.grad.float(), vi.grad.float(),

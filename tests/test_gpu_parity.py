@@ -70,6 +70,40 @@ def test_kv_proj_dx_dw_small(lvx, w_in_major):
     check_grad(dwv, dwv_ref, "dW_v")
 
 
+@pytest.mark.parametrize("w_in_major", [True, False])
+def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major):
+    from lv_xattn import ops
+    g = torch.Generator().manual_seed(6)
+    B, L, Dm, Hkv, D = 2, 301, 264, 4, 128          # ragged rows; 512 columns = two column tiles
+    x = (torch.randn(B, L, Dm, generator=g) * 0.5).bfloat16()
+    wk = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).bfloat16()
+    wv = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).bfloat16()
+    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).bfloat16()
+    eps = 1e-5
+    k_raw_ref, v_ref = orc.kv_project(x, wk, wv, Hkv)
+    k_raw_ref = k_raw_ref.bfloat16()
+    k_ref = orc.k_rms_norm(k_raw_ref, wn, eps)
+    wk_d, wv_d = (wk, wv) if w_in_major else (wk.t().contiguous(), wv.t().contiguous())
+    k, v, k_raw, rstd = ops.kv_proj(_dev(x), _dev(wk_d), _dev(wv_d), Hkv, w_in_major, k_norm_weight=_dev(wn),
+                                    eps=eps, for_backward=True)
+    k2, v2 = ops.kv_proj(_dev(x), _dev(wk_d), _dev(wv_d), Hkv, w_in_major, k_norm_weight=_dev(wn), eps=eps)
+    torch.cuda.synchronize()
+    check_grad(k, k_ref, "K (normed)")
+    check_grad(v, v_ref, "V")
+    check_grad(k_raw, k_raw_ref, "K (raw)")
+    assert torch.equal(k, k2) and torch.equal(v, v2)          # the optional outputs change nothing
+    r_ref = torch.rsqrt(k_raw_ref.float().pow(2).mean(-1) + eps).transpose(1, 2)     # [B, L, Hkv]
+    assert tuple(rstd.shape) == (B, L, Hkv)
+    assert ((rstd.cpu() - r_ref).abs() <= 1e-2 * r_ref).all()
+
+    dk = torch.randn(B, L, Hkv, D, generator=g).bfloat16().transpose(1, 2)
+    dx_ref, dw_ref = orc.k_rms_norm_backward(dk, k_raw.float().cpu(), wn, eps)
+    dk_raw, dw = ops.k_norm_bwd(_dev(dk.transpose(1, 2).contiguous()).transpose(1, 2), k_raw, rstd, _dev(wn))
+    torch.cuda.synchronize()
+    check_grad(dk_raw, dx_ref, "dK (raw)")
+    check_grad(dw, dw_ref, "dw_norm")
+
+
 # ------------------------------------------------------------------ row-wise kernels
 def test_merge_against_oracle(lvx):
     from lv_xattn import ops
@@ -271,6 +305,29 @@ def test_recompute_layer_autograd(lvx, name):
     check_grad(q.grad, ref["dq"], "dQ")
     check_grad(x.grad, ref["dx_vis"], "dX_vis")
     dwk_ref, dwv_ref = orc.dw_kv(t["x_vis"], ref["dk"].to(w.dtype), ref["dv"].to(w.dtype))
+    check_grad(wk.grad, dwk_ref, "dW_k")
+    check_grad(wv.grad, dwv_ref, "dW_v")
+
+
+def test_recompute_layer_with_k_norm_autograd(lvx):
+    w = orc.make_inputs(orc.workload("cfg2s"))
+    t = w.tensors
+    wn = (1.0 + 0.3 * torch.randn(w.D, generator=torch.Generator().manual_seed(9))).bfloat16()
+    ref = orc.layer_reference(w, k_norm_weight=wn, k_norm_eps=1e-5)
+    attention = lvx.create_attention_class("lv_xattn", rounds=w.rounds, weight_grads=True).apply
+    q = _dev(t["q"]).requires_grad_()
+    x = _dev(t["x_vis"]).requires_grad_()
+    wk = _dev(t["w_k"]).requires_grad_()
+    wv = _dev(t["w_v"]).requires_grad_()
+    wnd = _dev(wn).requires_grad_()
+    o = attention(q, x, wk, wv, w.Hkv, w.scale, None, wnd, 1e-5)
+    o.backward(_dev(t["do"]))
+    torch.cuda.synchronize()
+    check_o(o.detach(), ref["o"])
+    check_grad(q.grad, ref["dq"], "dQ")
+    check_grad(x.grad, ref["dx_vis"], "dX_vis")
+    check_grad(wnd.grad, ref["dw_norm"], "dw_norm")
+    dwk_ref, dwv_ref = orc.dw_kv(t["x_vis"], ref["dk_raw"].to(w.dtype), ref["dv"].to(w.dtype))
     check_grad(wk.grad, dwk_ref, "dW_k")
     check_grad(wv.grad, dwv_ref, "dW_v")
 

@@ -303,3 +303,35 @@ def test_backward_with_bias_against_autograd():
     assert (dq.double() - q.grad).abs().max() < 1e-4
     assert (dk.double() - k.grad).abs().max() < 1e-4
     assert (dv.double() - v.grad).abs().max() < 1e-4
+
+
+def test_k_rms_norm_against_library_class_and_hand_case():
+    # hand case: x = (3, 4, 0, 0), eps = 0 -> rms = sqrt(25/4) = 2.5 -> xh = (1.2, 1.6, 0, 0)
+    y = orc.k_rms_norm(torch.tensor([[3.0, 4.0, 0.0, 0.0]]), torch.tensor([1.0, 0.5, 2.0, 2.0]), eps=0.0)
+    assert torch.allclose(y, torch.tensor([[1.2, 0.8, 0.0, 0.0]]), atol=1e-6)
+    from transformers.models.mllama.modeling_mllama import MllamaTextRMSNorm
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 3, 17, 128, generator=g) * 1.7
+    norm = MllamaTextRMSNorm(128, eps=1e-5)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(128, generator=g))
+        assert torch.allclose(orc.k_rms_norm(x, norm.weight, 1e-5), norm(x), atol=1e-5, rtol=1e-5)
+
+
+def test_k_rms_norm_backward_against_autograd_and_finite_differences():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 2, 5, 128, generator=g, dtype=torch.float64).requires_grad_()
+    w = torch.randn(128, generator=g, dtype=torch.float64).requires_grad_()
+    dy = torch.randn(2, 2, 5, 128, generator=g, dtype=torch.float64)
+    y = w * x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5)
+    y.backward(dy)
+    dx, dw = orc.k_rms_norm_backward(dy, x.detach(), w.detach(), 1e-5)
+    assert torch.allclose(dx.double(), x.grad, atol=1e-5, rtol=1e-4)
+    assert torch.allclose(dw.double(), w.grad, atol=1e-4, rtol=1e-4)
+    # one directional finite difference in float64 through the oracle's forward
+    xd = x.detach()
+    u = torch.randn_like(xd)
+    h = 1e-3
+    f = lambda t: (orc.k_rms_norm(t.float(), w.detach().float(), 1e-5).double() * dy).sum()
+    fd = (f(xd + h * u) - f(xd - h * u)) / (2 * h)
+    assert abs(fd - (x.grad * u).sum()) < 2e-2 * max(1.0, abs(fd))
