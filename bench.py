@@ -118,7 +118,7 @@ def kernel_breakdown(layer, n_pairs, torch):
     o_p, l_p = torch.empty_like(o), torch.empty_like(L)
     delta = torch.empty_like(L)
     dq = torch.empty(B, Hq, Lq, D, dtype=torch.bfloat16, device=dev)
-    bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq), dtype=torch.uint8, device=dev)
+    bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, layer.mask), dtype=torch.uint8, device=dev)
     dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
     dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
     ops.bwd_preprocess(o, layer.do, delta)
@@ -179,7 +179,7 @@ def run_only(layer, which, n, torch):
         delta = torch.empty_like(L)
         ops.bwd_preprocess(o, layer.do, delta)
         dq = torch.empty_like(layer.q)
-        bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq), dtype=torch.uint8, device=dev)
+        bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, layer.mask), dtype=torch.uint8, device=dev)
         dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
         dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
         fn = lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask, workspace=bws)

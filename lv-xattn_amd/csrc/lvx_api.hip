@@ -239,7 +239,8 @@ static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
 // partial tiles into a scratch, rounded to bf16 afterwards.  Returns the number of
 // splits (1: none) and the tokens per split.
 static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_len) {
-    const int tiles = row_count > 256 ? (row_count + 511) / 512 : 1;
+    const int tile_rows = s->kv_start ? 256 : 512;      // as launch_gemm picks them
+    const int tiles = row_count > 256 ? (row_count + tile_rows - 1) / tile_rows : 1;
     const int wgs = s->B * s->Hq * tiles;
     const int blocks = (s->Lkv + 127) / 128;
     int ks = 1;
@@ -249,16 +250,42 @@ static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_le
     return (blocks + per - 1) / per;
 }
 
-size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
-    if (!s || row_count <= 0) return 0;
+// Regions of the backward workspace, in order: dS^T tiles; fp32 dK/dV scratch (split-steps mode
+// with bf16 outputs); row metadata records (2 floats per row and head); fp32 dQ partial sums
+// (split dQ contraction only); with an interval mask the live-tile tables (group hulls, runs
+// of live tiles per token block).  Every region is a multiple of 16 bytes.
+struct BwdWorkspace {
+    size_t ds, dkv, meta, dq32, hull, runs, total;
+    int n_tiles, group, n_groups;
+};
+
+static BwdWorkspace bwd_workspace(const lvx_attn_shape* s, int32_t row_count) {
+    BwdWorkspace w{};
     const size_t tokens = ((size_t)s->Lkv + 127) / 128 * 128;
     const size_t rows = ((size_t)row_count + 31) / 32 * 32;
-    // dS^T tiles, then fp32 dK/dV scratch for the split-steps mode with bf16 outputs, then the
-    // row metadata records (2 floats per row and head)
+    auto up16 = [](size_t n) { return (n + 15) / 16 * 16; };
+    w.n_tiles = (int)(rows / 32);
+    w.group = 8;                            // row tiles per M tile of the masked dQ GEMM (256 rows)
+    w.n_groups = (w.n_tiles + w.group - 1) / w.group;
+    size_t off = 0;
+    w.ds = off; off += (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t);
+    w.dkv = off; off += dkv_scratch_bytes(s);
+    w.meta = off; off += (size_t)s->B * s->Hq * rows * 2 * sizeof(float);
     int sl;
-    const size_t dq32 = dq_k_splits(s, row_count, &sl) > 1 ? (size_t)s->B * s->Hq * rows * s->D * sizeof(float) : 0;
-    return (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s) +
-           (size_t)s->B * s->Hq * rows * 2 * sizeof(float) + dq32;
+    w.dq32 = off;
+    if (dq_k_splits(s, row_count, &sl) > 1) off += (size_t)s->B * s->Hq * rows * s->D * sizeof(float);
+    if (s->kv_start) {
+        const size_t nkb = tokens / 128;
+        w.hull = off; off += up16((size_t)s->B * w.n_groups * 2 * sizeof(int32_t));
+        w.runs = off; off += (size_t)s->B * nkb * 8 * sizeof(int32_t);
+    }
+    w.total = off;
+    return w;
+}
+
+size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count) {
+    if (!s || row_count <= 0) return 0;
+    return bwd_workspace(s, row_count).total;
 }
 
 int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
@@ -303,13 +330,25 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.ws_ld = rows * 128;          // one token block: (rows / 32) tiles of 128 x 32
     p.ws_bh = tokens * rows;
 
+    const BwdWorkspace wsl = bwd_workspace(s, row_count);
+    char* const wsb = static_cast<char*>(workspace);
     {
-        float* meta = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                               (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s));
+        float* meta = reinterpret_cast<float*>(wsb + wsl.meta);
         MetaParams mp{lse, delta, meta, s->B, s->Hq, s->Lq, row_begin, row_begin + row_count, (int)(rows / 32), s->scale};
         hipError_t em = launch_bwd_meta(mp, st);
         if (em != hipSuccess) return static_cast<int>(em);
         p.meta = meta;
+    }
+    int32_t* hull = nullptr;
+    if (s->kv_start) {
+        // interval mask: token blocks skip the row tiles that see none of their tokens
+        hull = reinterpret_cast<int32_t*>(wsb + wsl.hull);
+        LiveParams lp{s->kv_len, s->kv_start, s->kv_end, hull, reinterpret_cast<int32_t*>(wsb + wsl.runs),
+                      s->B, s->Lq, s->Lkv, row_begin,
+                      row_begin + row_count, wsl.n_tiles, wsl.group, wsl.n_groups, p.n_kv_blocks};
+        hipError_t el = launch_bwd_live(lp, st);
+        if (el != hipSuccess) return static_cast<int>(el);
+        p.live_runs = lp.live_runs;
     }
 
     const int blocks = s->B * s->Hkv * p.n_kv_blocks;
@@ -324,8 +363,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         p.dkv_mode = 2;
         if (!dkv_accumulate) {
             // bf16 outputs: sum the splits in an fp32 scratch [2][B, Lkv, Hkv, D], round once afterwards
-            scratch = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                               (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t));
+            scratch = reinterpret_cast<float*>(wsb + wsl.dkv);
             FillParams f{reinterpret_cast<uint32_t*>(scratch), (int64_t)(dkv_scratch_bytes(s) / 16)};
             hipError_t ez = launch_zero(f, st);
             if (ez != hipSuccess) return static_cast<int>(ez);
@@ -366,14 +404,13 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.c_outer = dq->stride_b; g.c_inner = dq->stride_h;
     g.k_len = s->kv_len;
     g.a_tiled_m = (int)(rows / 32);
+    g.k_range = hull;            // [B][M tiles][2]: the group hulls are per M tile of this GEMM
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
     int split_len = 0;
     const int ks = dq_k_splits(s, row_count, &split_len);
     if (ks <= 1) return static_cast<int>(launch_gemm(g, true, true, st));
     // split contraction: zero the fp32 scratch, accumulate, round into dq
-    float* dq32 = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                           (size_t)s->B * s->Hq * tokens * rows * sizeof(uint16_t) + dkv_scratch_bytes(s) +
-                                           (size_t)s->B * s->Hq * rows * 2 * sizeof(float));
+    float* dq32 = reinterpret_cast<float*>(wsb + wsl.dq32);
     FillParams fz{reinterpret_cast<uint32_t*>(dq32), (int64_t)s->B * s->Hq * rows * s->D * (int64_t)sizeof(float) / 16};
     e = launch_zero(fz, st);
     if (e != hipSuccess) return static_cast<int>(e);

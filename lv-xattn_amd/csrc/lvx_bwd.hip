@@ -113,8 +113,23 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     // steps of this work-group: a contiguous range of the (head, row tile) list
     const int n_qtiles = (p.row_end - p.row_begin + BM - 1) / BM;
-    const int it_lo = sp * p.split_steps;
-    const int n_iter = (kvb < kv_len) ? max(0, min(p.split_steps, p.G * n_qtiles - it_lo)) : 0;
+    // with an interval mask only the listed runs of tiles are visited (kept in scalar
+    // registers), and the splits share that shorter walk evenly
+    int run_s[4] = {0, 0, 0, 0}, run_n[4] = {n_qtiles, 0, 0, 0};
+    int n_live = n_qtiles, split_steps = p.split_steps;
+    if (MASKED && p.live_runs) {
+        const int32_t* lr = p.live_runs + ((int64_t)b * p.n_kv_blocks + kblk) * 8;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            run_s[i] = __builtin_amdgcn_readfirstlane(lr[2 * i]);
+            run_n[i] = __builtin_amdgcn_readfirstlane(lr[2 * i + 1]);
+        }
+        n_live = run_n[0] + run_n[1] + run_n[2] + run_n[3];
+        split_steps = (p.G * n_live + p.q_splits - 1) / p.q_splits;
+    }
+    auto sel4 = [](int r, const int (&a)[4]) { return r == 0 ? a[0] : r == 1 ? a[1] : r == 2 ? a[2] : a[3]; };
+    const int it_lo = sp * split_steps;
+    const int n_iter = (kvb < kv_len) ? max(0, min(split_steps, p.G * n_live - it_lo)) : 0;
     const float c = p.scale_log2e;
 
     // global -> LDS is the P-waves' job (their step is the shorter one): P-wave w moves
@@ -151,7 +166,14 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     // The walk over (head of the group, 32-row tile): per-head base addresses are
     // re-derived only when the head changes, everything else advances by constants.
-    int cur_gi = it_lo / n_qtiles, cur_qt = it_lo % n_qtiles;
+    int cur_gi = 0, cur_run = 0, cur_qt = 0, cur_left = 1;    // cur_left: tiles left in the run, this one included
+    if (n_iter > 0) {
+        cur_gi = it_lo / n_live;
+        int idx = it_lo % n_live;
+        while (idx >= sel4(cur_run, run_n)) { idx -= sel4(cur_run, run_n); ++cur_run; }
+        cur_qt = sel4(cur_run, run_s) + idx;
+        cur_left = sel4(cur_run, run_n) - idx;
+    }
     const char* q_head = nullptr;      // Q, dO of (b, head)
     const char* do_head = nullptr;
     const float* meta_head = nullptr;  // metadata records of (b, head)
@@ -189,11 +211,15 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         dma16(do_head, row1 * dorow_b + ld_c1, slot + TILE_ELEMS * 2 + 1024);
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
-        if (++cur_qt == n_qtiles) {
-            cur_qt = 0;
+        ++cur_qt;
+        if (--cur_left > 0) return;
+        if (++cur_run == 4 || sel4(cur_run, run_n) == 0) {
+            cur_run = 0;
             if (++cur_gi == p.G) cur_gi = 0;
             enter_head();
         }
+        cur_qt = sel4(cur_run, run_s);
+        cur_left = sel4(cur_run, run_n);
     };
 
     // the finished dS^T tile goes to HBM as one contiguous 8 KB block

@@ -127,8 +127,14 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     uint16_t* const Cz = pr.C + zo * p.c_outer + zi * p.c_inner;
     int klen0 = pr.K[0];
     if (p.k_len) klen0 = min(klen0, p.k_len[zo]);
-    const int k_lo = ksp * p.k_split_len;          // 0 without a split
-    if (nks > 1) klen0 = max(0, min(klen0, k_lo + p.k_split_len) - k_lo);
+    int k_lo = 0;                                   // start of this work-group's k range
+    if (nks > 1) { k_lo = ksp * p.k_split_len; klen0 = min(klen0, k_lo + p.k_split_len); }
+    if (p.k_range) {
+        const int32_t* kr = p.k_range + ((int64_t)zo * p.tiles_m + tm) * 2;
+        k_lo = max(k_lo, kr[0]);
+        klen0 = min(klen0, kr[1]);
+    }
+    klen0 = max(0, klen0 - k_lo);
     const int s_lo = k_lo / BK;                    // first stage of this work-group's k range
     const int klen1 = pr.nseg > 1 ? pr.K[1] : 0;
 
@@ -365,7 +371,8 @@ hipError_t launch_cfg(GemmParams p, bool a_mcontig, bool b_ncontig, hipStream_t 
 }  // namespace
 
 // Work-group tile by shape: 256 x 256 in general; for a narrow C (N <= 128, the
-// dQ GEMM) 512 x 128, or 256 x 128 when there are not 512 rows.
+// dQ GEMM) 512 x 128, or 256 x 128 when there are not 512 rows or when M tiles have
+// their own contraction ranges (k_range is kept per 256 rows: finer ranges skip more).
 hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipStream_t st) {
     for (int i = 0; i < p.nprob; ++i) {
         const GemmProblem& pr = p.prob[i];
@@ -374,7 +381,7 @@ hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipS
         if (pr.nseg > 1 && (pr.lda[1] != pr.lda[0] || pr.ldb[1] != pr.ldb[0])) return hipErrorInvalidValue;
     }
     if (p.N > 128) return launch_cfg<2, 4, 4, 2, 4>(p, a_mcontig, b_ncontig, st);
-    if (p.M > 256) return launch_cfg<8, 1, 2, 4, 3>(p, a_mcontig, b_ncontig, st);
+    if (p.M > 256 && !p.k_range) return launch_cfg<8, 1, 2, 4, 3>(p, a_mcontig, b_ncontig, st);
     return launch_cfg<4, 2, 2, 2, 4>(p, a_mcontig, b_ncontig, st);
 }
 

@@ -80,7 +80,26 @@ struct BwdParams {
     int split_steps;           // steps (32-row tiles x heads of the group) per split
     int dkv_mode;              // 0: store bf16, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1)
     float scale, scale_log2e;
+    // Interval masks: the 32-row tiles each token block has to visit (the others see none of
+    // its tokens) as up to 4 runs of consecutive tiles, live_runs[(b * n_kv_blocks + block) * 8
+    // + 2 i + {0, 1}] = first tile and number of tiles of run i (0 tiles: unused).  Null: every tile.
+    const int32_t* live_runs;
 };
+
+// Which (token block, 32-row tile) pairs an interval mask leaves alive, at the granularity the
+// dQ GEMM needs: rows are taken in groups of `group` tiles (one M tile of that GEMM); a group's
+// hull is the smallest range of whole token blocks that holds every key some row of the group
+// sees, and all tiles of a group are alive for exactly the blocks of its hull.
+struct LiveParams {
+    const int32_t* kv_len;     // may be null
+    const int32_t* kv_start;
+    const int32_t* kv_end;
+    int32_t* hull;             // out: [B][n_groups][2] token range (multiples of 128), (0, 0) if empty
+    int32_t* live_runs;        // out, see BwdParams; a fifth run and later ones are merged into the
+                               // fourth together with the gaps between them (visiting more is harmless)
+    int B, Lq, Lkv, row_begin, row_end, n_tiles, group, n_groups, n_kv_blocks;
+};
+hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st);
 
 // Row metadata of the backward in the form its kernel consumes, one 256-byte
 // record per (b, h, 32-row tile of the window).
@@ -139,6 +158,9 @@ struct GemmParams {
     float norm_eps;
     uint16_t* c_raw;
     float* rstd;
+    // Per (outer batch index, M tile) contraction range of segment 0: k_range[(zo * tiles_m +
+    // tm) * 2 + {0, 1}] = first and one-past-last k (multiples of 128); null: all of K[0].
+    const int32_t* k_range;
     // Split contraction (single-segment problems): k_splits work-groups per C tile, each
     // contracting k_split_len values of k (a multiple of 128) and adding its partial tile
     // with fp32 atomics to the TRANSPOSED scratch c32[z * c32_batch + n * c32_ld + m] (zeroed

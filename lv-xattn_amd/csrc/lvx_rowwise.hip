@@ -7,6 +7,7 @@
 #include "lvx_kernels.hpp"
 
 #include <algorithm>
+#include <climits>
 
 namespace lvx {
 
@@ -131,6 +132,52 @@ __global__ __launch_bounds__(256) void bwd_meta_kernel(const MetaParams p) {
     o[32] = d * p.scale;
 }
 
+// One wave per (group of row tiles, b): the hull of the rows' key intervals in whole token blocks.
+__global__ __launch_bounds__(64) void bwd_hull_kernel(const LiveParams p) {
+    const int grp = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+    const int r0 = p.row_begin + grp * p.group * 32;
+    const int r1 = min(r0 + p.group * 32, p.row_end);
+    const int kv_len = p.kv_len ? min(p.kv_len[b], p.Lkv) : p.Lkv;
+    int lo = INT_MAX, hi = 0;
+    for (int r = r0 + lane; r < r1; r += 64) {
+        const int s = max(p.kv_start[(int64_t)b * p.Lq + r], 0);
+        const int e = min(p.kv_end[(int64_t)b * p.Lq + r], kv_len);
+        if (e > s) { lo = min(lo, s); hi = max(hi, e); }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        lo = min(lo, __shfl_xor(lo, o));
+        hi = max(hi, __shfl_xor(hi, o));
+    }
+    if (lane == 0) {
+        int32_t* h = p.hull + ((int64_t)b * p.n_groups + grp) * 2;
+        h[0] = hi > 0 ? (lo / 128) * 128 : 0;
+        h[1] = (hi + 127) / 128 * 128;
+    }
+}
+
+// One thread per (token block, b): the runs of consecutive row tiles whose group's hull holds the block.
+__global__ __launch_bounds__(64) void bwd_live_kernel(const LiveParams p) {
+    const int kblk = blockIdx.x * 64 + threadIdx.x, b = blockIdx.y;
+    if (kblk >= p.n_kv_blocks) return;
+    const int kvb = kblk * 128;
+    int32_t* out = p.live_runs + ((int64_t)b * p.n_kv_blocks + kblk) * 8;
+    int nr = 0, start = 0;
+    bool open = false;
+    for (int grp = 0; grp < p.n_groups; ++grp) {
+        const int32_t* h = p.hull + ((int64_t)b * p.n_groups + grp) * 2;
+        const bool live = h[0] <= kvb && kvb < h[1];
+        const int t0 = grp * p.group, t1 = min(t0 + p.group, p.n_tiles);
+        if (live) {
+            if (!open && nr < 4) { start = t0; ++nr; }
+            out[2 * (nr - 1)] = start;
+            out[2 * (nr - 1) + 1] = t1 - start;
+        }
+        open = live;
+    }
+    for (int i = nr; i < 4; ++i) { out[2 * i] = 0; out[2 * i + 1] = 0; }
+}
+
 __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
@@ -253,6 +300,15 @@ hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st) {
     const int64_t n = (int64_t)p.B * p.Hq * p.n_tiles * 32;
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(bwd_meta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st) {
+    if (p.B <= 0 || p.n_groups <= 0 || p.n_kv_blocks <= 0) return hipSuccess;
+    hipLaunchKernelGGL(bwd_hull_kernel, dim3(p.n_groups, p.B), dim3(64), 0, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), 0, st, p);
     return hipGetLastError();
 }
 

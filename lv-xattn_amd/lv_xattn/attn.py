@@ -167,7 +167,7 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     dv = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
-    ws = workspace("bwd_ds", (ops.bwd_workspace_bytes(q_, k_, max(r1 - r0 for r0, r1 in windows)),),
+    ws = workspace("bwd_ds", (ops.bwd_workspace_bytes(q_, k_, max(r1 - r0 for r0, r1 in windows), mask),),
                    torch.uint8, dev)
     if len(windows) == 1:
         r0, r1 = windows[0]

@@ -108,8 +108,10 @@ def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
     check(rc, "lvx_bwd_preprocess")
 
 
-def bwd_workspace_bytes(q, k, row_count: int) -> int:
-    s = _shape(q, k, 1.0, None)
+def bwd_workspace_bytes(q, k, row_count: int, mask: Optional[Mask] = None) -> int:
+    """Bytes lvx_bwd needs for `row_count` rows; pass the mask the call will use
+    (an interval mask adds its live-tile tables)."""
+    s = _shape(q, k, 1.0, mask)
     return int(load().lvx_bwd_workspace_bytes(C.byref(s), row_count))
 
 
@@ -118,7 +120,7 @@ def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=Non
         workspace: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
     """Writes dq (bf16) for the selected rows and writes (bf16) or accumulates
     (fp32) dk, dv at Hkv heads.  `workspace`: uint8 tensor of at least
-    bwd_workspace_bytes(q, k, row_count) bytes.  `bias` as in fwd (no gradient
+    bwd_workspace_bytes(q, k, row_count, mask) bytes.  `bias` as in fwd (no gradient
     is formed for it)."""
     s = _shape(q, k, scale, mask, bias)
     if row_count is None:
@@ -131,7 +133,7 @@ def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=Non
     if dk.dtype != want or dv.dtype != want or dk.shape != k.shape or dv.shape != k.shape:
         raise LvxError(f"dk/dv must be {want} tensors shaped like k")
     if workspace is None:
-        workspace = torch.empty(bwd_workspace_bytes(q, k, row_count), dtype=torch.uint8, device=q.device)
+        workspace = torch.empty(bwd_workspace_bytes(q, k, row_count, mask), dtype=torch.uint8, device=q.device)
     rc = load().lvx_bwd(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(dout)),
                         lse.data_ptr(), delta.data_ptr(), C.byref(t4(dq)), C.byref(t4(dk)), C.byref(t4(dv)),
                         1 if accumulate_dkv else 0, row_begin, row_count,
