@@ -1,0 +1,133 @@
+"""Forward and backward on randomly drawn small shapes and masks against the
+oracle: batch, head grouping, ragged lengths, rounds, launch mode, key-length
+and per-row interval masks (piecewise, with empty rows), strided inputs.  One
+case builds an interval mask under which a token block is seen by more than
+four separate runs of row groups (the backward keeps at most four runs per
+block and merges the rest)."""
+import random
+
+import pytest
+import torch
+
+from oracle import lvx_oracle as orc
+from parity import check_grad, check_lse, check_o
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def lvx():
+    import lv_xattn
+    from lv_xattn import _lib
+    _lib.load()
+    return lv_xattn
+
+
+def _piecewise_intervals(rng, B, Lq, Lkv, kv_len):
+    start = torch.zeros(B, Lq, dtype=torch.int32)
+    end = torch.zeros(B, Lq, dtype=torch.int32)
+    for b in range(B):
+        r = 0
+        while r < Lq:
+            n = rng.randint(1, max(1, Lq // 2))
+            kind = rng.random()
+            if kind < 0.2:
+                s = e = 0                                    # rows that see nothing
+            else:
+                s = rng.randint(0, kv_len[b] - 1)
+                e = rng.randint(s + 1, Lkv + 5)              # may reach past kv_len: clipped by it
+            start[b, r:r + n], end[b, r:r + n] = s, e
+            r += n
+    return start, end
+
+
+def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided):
+    D = 128
+    scale = rng.choice([D ** -0.5, 0.05, 0.2])
+    if strided:      # [B, S, H, D] memory viewed as [B, H, S, D]
+        q = torch.randn(B, Lq, Hq, D, generator=g).bfloat16().transpose(1, 2)
+        k = torch.randn(B, Lkv, Hkv, D, generator=g).bfloat16().transpose(1, 2)
+        v = torch.randn(B, Lkv, Hkv, D, generator=g).bfloat16().transpose(1, 2)
+    else:
+        q = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+        k = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
+        v = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
+    do = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+
+    kv_len = [Lkv] * B
+    mask, allowed = None, None
+    if mask_kind != "none":
+        kv_len = [rng.randint(1, Lkv) for _ in range(B)]
+        kl = torch.tensor(kv_len, dtype=torch.int32)
+        keys = torch.arange(Lkv)
+        allowed = (keys[None, :] < kl[:, None])[:, None, :].expand(B, Lq, Lkv).clone()
+        if mask_kind == "intervals":
+            start, end = _piecewise_intervals(rng, B, Lq, Lkv, kv_len)
+            allowed &= orc.interval_mask(start, end, Lkv)
+            mask = lvx.Mask(kl, start, end)
+        else:
+            mask = lvx.Mask(kl)
+    what = f"B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv} P{rounds} batched={batched} mask={mask_kind} strided={strided}"
+    print(what, flush=True)
+
+    o_ref, l_ref = orc.attention_dense(q, k, v, scale, allowed=allowed)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.bfloat16(), l_ref, scale, allowed=allowed)
+
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    _, _, _, o, L = lvx._attn_forward(qd, kd, vd, False, scale, None, rounds=rounds, mask=mask, batched=batched)
+    dq, dk, dv = lvx._attn_backward(dod, qd, kd, vd, o, L, False, scale, None, "flash", rounds=rounds,
+                                    mask=mask, batched=batched)
+    torch.cuda.synchronize()
+    check_o(o, o_ref, "O " + what)
+    check_lse(L, l_ref, "LSE " + what)
+    check_grad(dq, dq_ref, "dQ " + what)
+    check_grad(dk, dk_ref, "dK " + what)
+    check_grad(dv, dv_ref, "dV " + what)
+    dead = torch.isinf(l_ref).reshape(B, Hq, Lq)
+    assert (dq.float().cpu()[dead] == 0).all(), "dQ of rows that see nothing " + what
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shape_forward_backward(lvx, seed):
+    rng = random.Random(1000 + seed)
+    g = torch.Generator().manual_seed(2000 + seed)
+    B = rng.choice([1, 2, 3])
+    Hq, Hkv = rng.choice([(4, 4), (4, 2), (8, 2), (8, 1), (6, 3), (2, 1)])
+    Lq = rng.randint(1, 700)
+    Lkv = rng.randint(2, 900)
+    rounds = rng.choice([1, 2, 3, 5])
+    batched = rng.random() < 0.5
+    mask_kind = ["none", "kv_len", "intervals", "intervals"][seed % 4]
+    _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided=seed % 3 == 0)
+
+
+@pytest.mark.parametrize("batched", [True, False])
+def test_more_than_four_runs_of_live_row_groups(lvx, batched):
+    # 10 groups of 256 rows; group i sees only token block i % 2, so each of the two token
+    # blocks is alive for five separate runs of row tiles
+    B, Hq, Hkv, Lq, Lkv, D = 1, 2, 1, 2560, 256, 128
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
+    do = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+    grp = torch.arange(Lq) // 256
+    start = ((grp % 2) * 128 + 5).to(torch.int32)[None]
+    end = ((grp % 2) * 128 + 120).to(torch.int32)[None]
+    allowed = orc.interval_mask(start, end, Lkv)
+    scale = D ** -0.5
+    o_ref, l_ref = orc.attention_dense(q, k, v, scale, allowed=allowed)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.bfloat16(), l_ref, scale, allowed=allowed)
+    mask = lvx.Mask(None, start, end)
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    rounds = 1 if batched else 2
+    _, _, _, o, L = lvx._attn_forward(qd, kd, vd, False, scale, None, rounds=rounds, mask=mask, batched=batched)
+    dq, dk, dv = lvx._attn_backward(dod, qd, kd, vd, o, L, False, scale, None, "flash", rounds=rounds,
+                                    mask=mask, batched=batched)
+    torch.cuda.synchronize()
+    check_o(o, o_ref)
+    check_lse(L, l_ref)
+    check_grad(dq, dq_ref, "dQ")
+    check_grad(dk, dk_ref, "dK")
+    check_grad(dv, dv_ref, "dV")
