@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes moved by one lvx_bwd call at cfg2 (zero + dK/dV kernel + 2 casts + dQ GEMM), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy (profiles/cfg2_bwd_hbm_traffic.md)
-BWD_TRAFFIC_BYTES = {"cfg2": 4.48e9}
+BWD_TRAFFIC_BYTES = {"cfg2": 4.41e9}
 
 
 def flops(w, n_pairs):
