@@ -150,6 +150,11 @@ int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_
  * (test_llama3.py:395-398) run in forward and again in backward (:197, :235).
  * w_in_major != 0: W is [Dm, N] row-major;  w_in_major == 0: W is [N, Dm]
  * row-major (torch.nn.Linear.weight).  ld* are row strides in elements.
+ * w_v and v_out may both be null: a single projection, which with
+ * lvx_kv_proj_norm is the text side of `project`,
+ * `query_states = self.q_norm(self.q_proj(hidden_states))` (test_llama3.py:390-393).
+ * The same holds for the second operand pair of lvx_dx_vis (dv, w_v) and of
+ * lvx_dw_kv (dv, dw_v).
  */
 int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw,
                 int32_t w_in_major, void* k_out, void* v_out, int64_t ldkv,

@@ -466,15 +466,19 @@ static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void*
                         const void* k_norm_w, float eps, void* k_raw, float* k_rstd, void* stream) {
     LVX_TRY(check_gemm_ptr(x, ldx));
     LVX_TRY(check_gemm_ptr(w_k, ldw));
-    LVX_TRY(check_gemm_ptr(w_v, ldw));
     LVX_TRY(check_gemm_ptr(k_out, ldkv));
-    LVX_TRY(check_gemm_ptr(v_out, ldkv));
+    if (!w_v != !v_out) return LVX_ERR_NULL;       // both or neither
+    const int np = w_v ? 2 : 1;                    // one projection only: the Q side
+    if (np == 2) {
+        LVX_TRY(check_gemm_ptr(w_v, ldw));
+        LVX_TRY(check_gemm_ptr(v_out, ldkv));
+    }
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (ldx < Dm || ldkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
     const void* w[2] = {w_k, w_v};
     void* c[2] = {k_out, v_out};
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < np; ++i) {
         GemmProblem& pr = g.prob[i];
         pr.A[0] = static_cast<const uint16_t*>(x); pr.lda[0] = ldx;
         pr.Bm[0] = static_cast<const uint16_t*>(w[i]); pr.ldb[0] = ldw;
@@ -492,7 +496,7 @@ static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void*
         g.c_raw = static_cast<uint16_t*>(k_raw);
         g.rstd = k_rstd;
     }
-    fill_grid(g, M, N, 2);
+    fill_grid(g, M, N, np);
     return static_cast<int>(launch_gemm(g, false, w_in_major != 0, static_cast<hipStream_t>(stream)));
 }
 
@@ -537,10 +541,13 @@ int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk,
 int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v, int64_t ldw,
                int32_t w_in_major, void* dx, int64_t lddx, int32_t M, int32_t Dm, int32_t N, void* stream) {
     LVX_TRY(check_gemm_ptr(dk, lddkv));
-    LVX_TRY(check_gemm_ptr(dv, lddkv));
     LVX_TRY(check_gemm_ptr(w_k, ldw));
-    LVX_TRY(check_gemm_ptr(w_v, ldw));
     LVX_TRY(check_gemm_ptr(dx, lddx));
+    if (!dv != !w_v) return LVX_ERR_NULL;          // both or neither
+    if (dv) {
+        LVX_TRY(check_gemm_ptr(dv, lddkv));
+        LVX_TRY(check_gemm_ptr(w_v, ldw));
+    }
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (lddkv < N || lddx < Dm || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
@@ -549,7 +556,7 @@ int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, c
     pr.lda[0] = pr.lda[1] = lddkv;
     pr.Bm[0] = static_cast<const uint16_t*>(w_k); pr.Bm[1] = static_cast<const uint16_t*>(w_v);
     pr.ldb[0] = pr.ldb[1] = ldw;
-    pr.K[0] = pr.K[1] = N; pr.nseg = 2;
+    pr.K[0] = N; pr.K[1] = dv ? N : 0; pr.nseg = dv ? 2 : 1;
     pr.C = static_cast<uint16_t*>(dx); pr.ldc = lddx;
     fill_grid(g, M, Dm, 1);
     // B[k = n][col = dm]: W [Dm][N] has k contiguous, W [N][Dm] has the column contiguous
@@ -560,15 +567,19 @@ int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_
               int64_t ldw, int32_t w_in_major, int32_t M, int32_t Dm, int32_t N, void* stream) {
     LVX_TRY(check_gemm_ptr(x, ldx));
     LVX_TRY(check_gemm_ptr(dk, lddkv));
-    LVX_TRY(check_gemm_ptr(dv, lddkv));
     LVX_TRY(check_gemm_ptr(dw_k, ldw));
-    LVX_TRY(check_gemm_ptr(dw_v, ldw));
+    if (!dv != !dw_v) return LVX_ERR_NULL;         // both or neither
+    const int np = dv ? 2 : 1;
+    if (np == 2) {
+        LVX_TRY(check_gemm_ptr(dv, lddkv));
+        LVX_TRY(check_gemm_ptr(dw_v, ldw));
+    }
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (ldx < Dm || lddkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
     const void* d[2] = {dk, dv};
     void* c[2] = {dw_k, dw_v};
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < np; ++i) {
         GemmProblem& pr = g.prob[i];
         if (w_in_major) {   // dW [Dm][N] = X^T dK
             pr.A[0] = static_cast<const uint16_t*>(x); pr.lda[0] = ldx;
@@ -580,8 +591,8 @@ int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_
         pr.K[0] = M; pr.nseg = 1;
         pr.C = static_cast<uint16_t*>(c[i]); pr.ldc = ldw;
     }
-    if (w_in_major) fill_grid(g, Dm, N, 2);
-    else fill_grid(g, N, Dm, 2);
+    if (w_in_major) fill_grid(g, Dm, N, np);
+    else fill_grid(g, N, Dm, np);
     return static_cast<int>(launch_gemm(g, true, true, static_cast<hipStream_t>(stream)));
 }
 

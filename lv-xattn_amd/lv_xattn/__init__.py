@@ -6,10 +6,11 @@ device work is done by hand-written gfx950 kernels in liblvx.so.
 from .attn import _attn_forward, _attn_backward, Mask, q_block_bounds
 from .async_communication import (initialize_distributed, reset_global_memory_buffer,
                                   get_sequence_parallel_group)
-from .autograd import create_attention_class, create_attention_class_save_qkv, KVProjection
+from .autograd import (create_attention_class, create_attention_class_save_qkv, create_q_projection_class,
+                       KVProjection)
 
 __all__ = [
     "_attn_forward", "_attn_backward", "initialize_distributed", "reset_global_memory_buffer",
     "get_sequence_parallel_group", "Mask", "q_block_bounds",
-    "create_attention_class", "create_attention_class_save_qkv", "KVProjection",
+    "create_attention_class", "create_attention_class_save_qkv", "create_q_projection_class", "KVProjection",
 ]

@@ -126,3 +126,32 @@ def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = 
             return (dq, dx, dwk, dwv, None, None, None, dwn, None, None) + (None,) * ctx.n_bias
 
     return _attention
+
+
+def create_q_projection_class(w_in_major: bool = True, weight_grads: bool = True):
+    """apply(x, w_q, n_heads, q_norm_weight, eps) -> q [B, Hq, Lq, D]
+
+    The text side of the reference's `project` (test_llama3.py:390-393),
+    Q = q_norm(X W_q), with the reference's recompute discipline
+    (test_llama3.py:184-243: only the layer input is kept): forward saves
+    (x, w_q, norm weight); backward re-runs the fused GEMM to get the raw
+    projection and r, goes back through the norm, then dX = dQ_raw W_q^T and
+    dW_q = X^T dQ_raw."""
+
+    class _q_projection(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, w_q, n_heads, q_norm_weight, eps=1e-5):
+            ctx.save_for_backward(x, w_q, q_norm_weight)
+            ctx.n_heads, ctx.eps = n_heads, eps
+            return ops.q_proj(x, w_q, n_heads, w_in_major, q_norm_weight, eps)
+
+        @staticmethod
+        def backward(ctx, dq):
+            x, w_q, wn = ctx.saved_tensors
+            _, q_raw, rstd = ops.q_proj(x, w_q, ctx.n_heads, w_in_major, wn, ctx.eps, for_backward=True)
+            dq_tm = dq if dq.transpose(1, 2).is_contiguous() else dq.transpose(1, 2).contiguous().transpose(1, 2)
+            dq_raw, dwn = ops.k_norm_bwd(dq_tm, q_raw, rstd, wn, want_dw=weight_grads)
+            dx, dw = ops.q_proj_bwd(x, dq_raw, w_q, w_in_major, want_dw=weight_grads)
+            return dx, dw, None, (dwn.to(wn.dtype) if dwn is not None else None), None
+
+    return _q_projection

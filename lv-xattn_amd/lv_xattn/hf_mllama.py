@@ -33,7 +33,7 @@ from typing import Optional
 import torch
 
 from ._lib import LvxError
-from .autograd import create_attention_class, create_attention_class_save_qkv
+from .autograd import create_attention_class, create_attention_class_save_qkv, create_q_projection_class
 
 NAME = "lv_xattn"
 _attention = None
@@ -99,15 +99,19 @@ def _recompute_forward(self, hidden_states, cross_attention_states=None, past_ke
         return self._lvx_stock_forward(hidden_states, cross_attention_states, past_key_values,
                                        attention_mask, use_cache, **kwargs)
     bsz, q_len, _ = hidden_states.size()
-    query = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-    query = self.q_norm(query)
     dropout = self.dropout if self.training else 0.0
-    if not (query.is_cuda and query.dtype == torch.bfloat16 and self.head_dim == 128 and dropout == 0.0):
+    if not (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and self.head_dim == 128
+            and dropout == 0.0):
         raise LvxError("lv_xattn cross-attention needs bf16 tensors on the GPU, head_dim 128 and no dropout")
     key = (self._lvx_rounds, self._lvx_batched, self._lvx_weight_grads)
     if key not in _recompute:
         _recompute[key] = create_attention_class("lv_xattn", rounds=key[0], batched=key[1],
                                                  weight_grads=key[2], w_in_major=False).apply
+    if ("q", key[2]) not in _recompute:
+        _recompute[("q", key[2])] = create_q_projection_class(w_in_major=False, weight_grads=key[2]).apply
+    # q_proj + q_norm in the fused GEMM; like K/V, Q is recomputed from the layer input in backward
+    query = _recompute[("q", key[2])](hidden_states.contiguous(), self.q_proj.weight, self.num_heads,
+                                      self.q_norm.weight, self.q_norm.variance_epsilon)
     mask = kwargs.get("lvx_mask")
     bias = []
     if mask is None and attention_mask is not None:

@@ -233,6 +233,64 @@ def k_norm_bwd(dk, k_raw, k_rstd, k_norm_weight, want_dw: bool = True):
     return out.view(B, Lkv, Hkv, D).transpose(1, 2), dw
 
 
+def q_proj(x, w_q, n_heads: int, w_in_major: bool = True, q_norm_weight: Optional[torch.Tensor] = None,
+           eps: float = 1e-5, for_backward: bool = False):
+    """Q = q_norm(X W_q) (test_llama3.py:390-393 in the reference): the K side of
+    kv_proj on its own.  x [B, Lq, Dm]; returns a [B, Hq, Lq, D] view of
+    [B, Lq, Hq, D] memory (and, with `for_backward`, the raw projection and r)."""
+    B, Lq, Dm = x.shape
+    N = w_q.shape[1] if w_in_major else w_q.shape[0]
+    xp, M, ldx = _rows2d(x, "x")
+    wp, _, ldw = _rows2d(w_q, "w_q")
+    D = N // n_heads
+    q = torch.empty(B, Lq, N, dtype=torch.bfloat16, device=x.device)
+
+    def heads(t):
+        return t.view(B, Lq, n_heads, D).transpose(1, 2)
+
+    if q_norm_weight is None:
+        if for_backward:
+            raise LvxError("for_backward only applies with q_norm_weight")
+        rc = load().lvx_kv_proj(xp, ldx, wp, None, ldw, 1 if w_in_major else 0, q.data_ptr(), None, N,
+                                M, Dm, N, stream_ptr())
+        check(rc, "lvx_kv_proj")
+        return heads(q)
+    wn = _norm_weight(q_norm_weight, D, x.device)
+    raw = torch.empty_like(q) if for_backward else None
+    rstd = torch.empty(B, Lq, n_heads, dtype=torch.float32, device=x.device) if for_backward else None
+    rc = load().lvx_kv_proj_norm(xp, ldx, wp, None, ldw, 1 if w_in_major else 0, q.data_ptr(), None, N,
+                                 M, Dm, N, wn.data_ptr(), float(eps),
+                                 raw.data_ptr() if for_backward else None,
+                                 rstd.data_ptr() if for_backward else None, stream_ptr())
+    check(rc, "lvx_kv_proj_norm")
+    if for_backward:
+        return heads(q), heads(raw), rstd
+    return heads(q)
+
+
+def q_proj_bwd(x, dq_raw, w_q, w_in_major: bool = True, want_dw: bool = True):
+    """(dX, dW_q) of Q_raw = X W_q from dq_raw ([B, Hq, Lq, D] view of
+    [B, Lq, Hq, D] memory)."""
+    B, Hq, Lq, D = dq_raw.shape
+    N = Hq * D
+    d2 = _token_major(dq_raw, "dq_raw")
+    Dm = w_q.shape[0] if w_in_major else w_q.shape[1]
+    wp, _, ldw = _rows2d(w_q, "w_q")
+    xp, M, ldx = _rows2d(x, "x")
+    dx = torch.empty(B, Lq, Dm, dtype=torch.bfloat16, device=x.device)
+    rc = load().lvx_dx_vis(d2.data_ptr(), None, N, wp, None, ldw, 1 if w_in_major else 0, dx.data_ptr(), Dm,
+                           M, Dm, N, stream_ptr())
+    check(rc, "lvx_dx_vis")
+    dw = None
+    if want_dw:
+        shape = (Dm, N) if w_in_major else (N, Dm)
+        dw = torch.empty(*shape, dtype=torch.bfloat16, device=x.device)
+        rc = load().lvx_dw_kv(xp, ldx, d2.data_ptr(), None, N, dw.data_ptr(), None, shape[1],
+                              1 if w_in_major else 0, M, Dm, N, stream_ptr())
+        check(rc, "lvx_dw_kv")
+    return dx, dw
+
+
 def _token_major(t: torch.Tensor, name: str) -> torch.Tensor:
     """[B, Hkv, Lkv, D] view whose memory is [B, Lkv, Hkv, D] -> [B*Lkv, Hkv*D]."""
     tm = t.transpose(1, 2)

@@ -113,6 +113,16 @@ def test_other_entry_points_reject_bad_arguments(lib):
     assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, None) == -1
     assert lib.lvx_dx_vis(0x1000, 0x1100, 256, 0x2000, 0x3000, 250, 1, 0x4000, 512, 100, 512, 256, None) == -2
     assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, 0x3000, 128, 1, 100, 512, 256, None) == -3
+    # the second operand pair is optional (single projection) but must be given or omitted as a pair
+    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, None, 256, 100, 512, 256, None) == -1
+    assert lib.lvx_dx_vis(0x1000, None, 256, 0x2000, 0x3000, 256, 1, 0x4000, 512, 100, 512, 256, None) == -1
+    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, None, 256, 1, 100, 512, 256, None) == -1
+    # the fused norm needs whole heads of 128 columns and its weight
+    assert lib.lvx_kv_proj_norm(0x1000, 512, 0x2000, 0x3000, 192, 1, 0x4000, 0x5000, 192, 100, 512, 192,
+                                0x6000, 1e-5, None, None, None) == -4
+    assert lib.lvx_kv_proj_norm(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256,
+                                None, 1e-5, None, None, None) == -1
+    assert lib.lvx_k_norm_bwd(0x1000, 256, 0x2000, 256, None, 0x3000, 0x4000, 256, None, 100, 256, None) == -1
 
 
 def test_missing_library_fails_loudly(monkeypatch):

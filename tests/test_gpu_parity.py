@@ -104,6 +104,36 @@ def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major):
     check_grad(dw, dw_ref, "dw_norm")
 
 
+@pytest.mark.parametrize("w_in_major", [True, False])
+def test_q_projection_with_q_norm_autograd(lvx, w_in_major):
+    # the text side of `project`: Q = q_norm(X W_q), recomputed in backward
+    g = torch.Generator().manual_seed(8)
+    B, L, Dm, Hq, D = 2, 203, 328, 3, 128
+    x = (torch.randn(B, L, Dm, generator=g) * 0.5).bfloat16()
+    wq = (torch.randn(Dm, Hq * D, generator=g) * 0.1).bfloat16()
+    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).bfloat16()
+    dq = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    q_raw_ref, _ = orc.kv_project(x, wq, wq, Hq)
+    q_raw_ref = q_raw_ref.bfloat16()
+    q_ref = orc.k_rms_norm(q_raw_ref, wn, 1e-5)
+    dq_raw_ref, dwn_ref = orc.k_rms_norm_backward(dq, q_raw_ref, wn, 1e-5)
+    dx_ref = orc.dx_vis(dq_raw_ref.bfloat16(), torch.zeros_like(dq_raw_ref), wq, wq)
+    dw_ref, _ = orc.dw_kv(x, dq_raw_ref.bfloat16(), torch.zeros_like(dq_raw_ref))
+
+    proj = lvx.create_q_projection_class(w_in_major=w_in_major).apply
+    xd = _dev(x).requires_grad_()
+    wd = _dev(wq if w_in_major else wq.t().contiguous()).requires_grad_()
+    wnd = _dev(wn).requires_grad_()
+    q = proj(xd, wd, Hq, wnd, 1e-5)
+    assert tuple(q.shape) == (B, Hq, L, D)
+    q.backward(_dev(dq))
+    torch.cuda.synchronize()
+    check_grad(q.detach(), q_ref, "Q")
+    check_grad(xd.grad, dx_ref, "dX")
+    check_grad(wd.grad if w_in_major else wd.grad.t(), dw_ref, "dW_q")
+    check_grad(wnd.grad, dwn_ref, "dw_norm")
+
+
 # ------------------------------------------------------------------ row-wise kernels
 def test_merge_against_oracle(lvx):
     from lv_xattn import ops
