@@ -51,7 +51,7 @@ constexpr int BM = 32;        // text rows per step
 constexpr int NT = 512;       // threads per work-group
 constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row]
 
-// LDS map (uint16 units): four (Q | dO) tile pairs, unpadded; two dS^T tiles; two P hand-over buffers
+// LDS map (uint16 units): a ring of five (Q | dO) tile pairs, unpadded; two dS^T tiles; two P hand-over buffers
 constexpr int TILE_ELEMS = BM * D;             // one Q or dO tile (8 KiB)
 constexpr int QD_ELEMS = 2 * TILE_ELEMS;
 constexpr int NQD = 5;
