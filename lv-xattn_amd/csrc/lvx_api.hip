@@ -332,9 +332,25 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
 
     const BwdWorkspace wsl = bwd_workspace(s, row_count);
     char* const wsb = static_cast<char*>(workspace);
+    // how the launch is shaped decides which fp32 scratches it accumulates into; the
+    // metadata kernel zeroes them on its way
+    const int blocks = s->B * s->Hkv * p.n_kv_blocks;
+    const int steps = p.G * (int)(rows / 32);
+    p.q_splits = choose_q_splits(blocks, steps);
+    p.split_steps = (steps + p.q_splits - 1) / p.q_splits;
+    p.total_wg = blocks * p.q_splits;
+    p.dkv_mode = p.q_splits > 1 ? 2 : (dkv_accumulate ? 1 : 0);
+    float* const scratch = (p.q_splits > 1 && !dkv_accumulate) ? reinterpret_cast<float*>(wsb + wsl.dkv) : nullptr;
+    int split_len = 0;
+    const int ks = dq_k_splits(s, row_count, &split_len);
+    float* const dq32 = ks > 1 ? reinterpret_cast<float*>(wsb + wsl.dq32) : nullptr;
     {
         float* meta = reinterpret_cast<float*>(wsb + wsl.meta);
         MetaParams mp{lse, delta, meta, s->B, s->Hq, s->Lq, row_begin, row_begin + row_count, (int)(rows / 32), s->scale};
+        mp.zero_dst[0] = reinterpret_cast<uint32_t*>(scratch);
+        mp.zero_n16[0] = scratch ? (int64_t)(dkv_scratch_bytes(s) / 16) : 0;
+        mp.zero_dst[1] = reinterpret_cast<uint32_t*>(dq32);
+        mp.zero_n16[1] = dq32 ? (int64_t)s->B * s->Hq * rows * s->D * (int64_t)sizeof(float) / 16 : 0;
         hipError_t em = launch_bwd_meta(mp, st);
         if (em != hipSuccess) return static_cast<int>(em);
         p.meta = meta;
@@ -351,26 +367,13 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         p.live_runs = lp.live_runs;
     }
 
-    const int blocks = s->B * s->Hkv * p.n_kv_blocks;
-    const int steps = p.G * (int)(rows / 32);
-    p.q_splits = choose_q_splits(blocks, steps);
-    p.split_steps = (steps + p.q_splits - 1) / p.q_splits;
-    p.total_wg = blocks * p.q_splits;
-    p.dkv_mode = dkv_accumulate ? 1 : 0;
-    float* scratch = nullptr;
     const int64_t dkv_elems = (int64_t)s->B * s->Lkv * s->Hkv * s->D;
-    if (p.q_splits > 1) {
-        p.dkv_mode = 2;
-        if (!dkv_accumulate) {
-            // bf16 outputs: sum the splits in an fp32 scratch [2][B, Lkv, Hkv, D], round once afterwards
-            scratch = reinterpret_cast<float*>(wsb + wsl.dkv);
-            FillParams f{reinterpret_cast<uint32_t*>(scratch), (int64_t)(dkv_scratch_bytes(s) / 16)};
-            hipError_t ez = launch_zero(f, st);
-            if (ez != hipSuccess) return static_cast<int>(ez);
-            p.dk = scratch;
-            p.dv = scratch + dkv_elems;
-            p.dks = p.dvs = Strides3{(int64_t)s->Lkv * s->Hkv * s->D, (int64_t)s->D, (int64_t)s->Hkv * s->D};
-        }
+    if (scratch) {
+        // bf16 outputs, several work-groups per token block: sum in the fp32 scratch
+        // [2][B, Lkv, Hkv, D], round once afterwards
+        p.dk = scratch;
+        p.dv = scratch + dkv_elems;
+        p.dks = p.dvs = Strides3{(int64_t)s->Lkv * s->Hkv * s->D, (int64_t)s->D, (int64_t)s->Hkv * s->D};
     }
     hipError_t e = launch_bwd(p, s->kv_start != nullptr, st);
     if (e != hipSuccess) return static_cast<int>(e);
@@ -406,14 +409,8 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.a_tiled_m = (int)(rows / 32);
     g.k_range = hull;            // [B][M tiles][2]: the group hulls are per M tile of this GEMM
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
-    int split_len = 0;
-    const int ks = dq_k_splits(s, row_count, &split_len);
     if (ks <= 1) return static_cast<int>(launch_gemm(g, true, true, st));
-    // split contraction: zero the fp32 scratch, accumulate, round into dq
-    float* dq32 = reinterpret_cast<float*>(wsb + wsl.dq32);
-    FillParams fz{reinterpret_cast<uint32_t*>(dq32), (int64_t)s->B * s->Hq * rows * s->D * (int64_t)sizeof(float) / 16};
-    e = launch_zero(fz, st);
-    if (e != hipSuccess) return static_cast<int>(e);
+    // split contraction: accumulate in the (already zeroed) fp32 scratch, round into dq
     g.k_splits = ks; g.k_split_len = split_len;
     g.c32 = dq32; g.c32_batch = (int64_t)row_count * s->D; g.c32_ld = row_count;   // [B * Hq][D][row_count]
     e = launch_gemm(g, true, true, st);

@@ -109,6 +109,11 @@ struct MetaParams {
     float* out;
     int B, Hq, Lq, row_begin, row_end, n_tiles;
     float scale;
+    // up to two regions the same launch zero-fills (the fp32 scratches the call accumulates
+    // into); dst 16-byte aligned, n16 = number of 16-byte chunks, 0: none
+    uint32_t* zero_dst[2];
+    int64_t zero_n16[2];
+    int meta_blocks;           // filled by the launcher: blocks [0, meta_blocks) write records
 };
 
 struct FillParams {

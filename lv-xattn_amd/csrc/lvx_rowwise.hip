@@ -118,6 +118,15 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
 // window (so that P = exp2(x - inf) = 0 there), and delta * scale (0 past the
 // window), grouped per 32-row tile so that one 256-byte load fetches a tile's lot.
 __global__ __launch_bounds__(256) void bwd_meta_kernel(const MetaParams p) {
+    if ((int)blockIdx.x >= p.meta_blocks) {   // the other blocks of the launch zero the scratches
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const int64_t first = (int64_t)(blockIdx.x - p.meta_blocks) * 256 + threadIdx.x;
+        const int64_t stride = (int64_t)(gridDim.x - p.meta_blocks) * 256;
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            for (int64_t i = first; i < p.zero_n16[r]; i += stride) reinterpret_cast<u32x4*>(p.zero_dst[r])[i] = z;
+        return;
+    }
     const int rows_pad = p.n_tiles * 32;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (int64_t)p.B * p.Hq * rows_pad) return;
@@ -296,10 +305,14 @@ hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     return hipGetLastError();
 }
 
-hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st) {
+hipError_t launch_bwd_meta(const MetaParams& p0, hipStream_t st) {
+    MetaParams p = p0;
     const int64_t n = (int64_t)p.B * p.Hq * p.n_tiles * 32;
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(bwd_meta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p);
+    const int64_t z = p.zero_n16[0] + p.zero_n16[1];
+    if (n == 0 && z == 0) return hipSuccess;
+    p.meta_blocks = (int)((n + 255) / 256);
+    const int zero_blocks = (int)std::min<int64_t>((z + 255) / 256, 2048);
+    hipLaunchKernelGGL(bwd_meta_kernel, dim3((unsigned)(p.meta_blocks + zero_blocks)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
