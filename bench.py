@@ -59,7 +59,7 @@ class Layer:
             kv_len = torch.tensor(w.kv_len, dtype=torch.int32) if w.kv_len else None
             self.mask = lv_xattn.Mask(kv_len, t.get("kv_start"), t.get("kv_end")).to(dev)
         B, Hq, Lq, D = self.q.shape
-        self.o_in = torch.zeros(B, Hq, Lq, D, dtype=torch.bfloat16, device=dev)
+        self.o_in = torch.zeros(B, Hq, Lq, D, dtype=w.dtype, device=dev)
         self.l_in = torch.full((B * Hq, Lq), float("-inf"), device=dev)
         self.batched = mode == "batched"
         self.out = {}
@@ -117,9 +117,9 @@ def kernel_breakdown(layer, n_pairs, torch):
     dev = layer.q.device
     o_p, l_p = torch.empty_like(o), torch.empty_like(L)
     delta = torch.empty_like(L)
-    dq = torch.empty(B, Hq, Lq, D, dtype=torch.bfloat16, device=dev)
+    dq = torch.empty(B, Hq, Lq, D, dtype=w.dtype, device=dev)
     bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, layer.mask), dtype=torch.uint8, device=dev)
-    dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+    dk = torch.empty(B, Lkv, Hkv, D, dtype=w.dtype, device=dev).transpose(1, 2)
     dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
     ops.bwd_preprocess(o, layer.do, delta)
     res = {}
@@ -180,7 +180,7 @@ def run_only(layer, which, n, torch):
         ops.bwd_preprocess(o, layer.do, delta)
         dq = torch.empty_like(layer.q)
         bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, layer.mask), dtype=torch.uint8, device=dev)
-        dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+        dk = torch.empty(B, Lkv, Hkv, D, dtype=w.dtype, device=dev).transpose(1, 2)
         dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
         fn = lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask, workspace=bws)
     elif which == "kv_proj":
@@ -243,6 +243,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--mode", default="batched", choices=["batched", "rounds"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--only", choices=["fwd", "bwd", "kv_proj", "dx_vis", "copy"],
@@ -260,6 +261,9 @@ def main():
     _lib.load()
     dev = "cuda:0"
     w = orc.make_inputs(orc.workload(a.workload))
+    if a.dtype == "fp16":      # the reference's element type; same kernels, fp16 MFMA
+        w.dtype = torch.float16
+        w.tensors = {n: (t.to(torch.float16) if t.is_floating_point() else t) for n, t in w.tensors.items()}
     npairs = orc.n_pairs(w)
     f = flops(w, npairs)
     step_flops = f["fwd"] + f["bwd"] + 3 * f["proj"]    # projection, re-projection, dX_vis
@@ -282,7 +286,7 @@ def main():
         "metric": "cross-attn fwd+bwd TFLOP/s @ Llama-3.2-11B-V shape, 1 GPU; % bf16 MFMA peak",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic (seeded N(0,1) Q/dO, N(0,0.02) X_vis/W), random weights",
+        "dtype": a.dtype, "data": "synthetic (seeded N(0,1) Q/dO, N(0,0.02) X_vis/W), random weights",
         "config": {
             "workload": f"{w.name}: B{w.B} Hq{w.Hq} Hkv{w.Hkv} D{w.D} Lq{w.Lq}={w.rounds}x{-(-w.Lq // w.rounds)} "
                         f"Lkv{w.Lkv} Dm{w.Dm}; K/V projection + {w.rounds}-round fwd + merge + K/V re-projection "
@@ -295,7 +299,7 @@ def main():
         kb = kernel_breakdown(layer, npairs, torch)
         out["kernels"] = kb
         dom = kb["bwd_all_rounds_one_launch"]
-        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel + zero_kernel + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
+        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel (incl. scratch zero-fill) + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
                            "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
                            "traffic": BWD_TRAFFIC_BYTES.get(w.name) if a.mode == "batched" else None,

@@ -9,7 +9,7 @@
  *     allocates nothing, keeps no pointer after a call returns and never
  *     synchronises: all work is queued on `stream` (a hipStream_t, NULL = the
  *     default stream);
- *   - 16-bit tensors are bf16; strides are in ELEMENTS, the last (head_dim)
+ *   - 16-bit tensors are bf16 or fp16 (one type per call, "16-bit" below); strides are in ELEMENTS, the last (head_dim)
  *     stride is 1, every other stride is a multiple of 8 and every base pointer
  *     is 16-byte aligned;
  *   - q-like tensors are indexed [batch, q_head, text_row, d], kv-like tensors
@@ -40,19 +40,20 @@ extern "C" {
 #define LVX_ERR_ALIGN (-2)       /* pointer not 16-byte aligned / stride not a multiple of 8 */
 #define LVX_ERR_SHAPE (-3)       /* non-positive or inconsistent sizes, bad row window */
 #define LVX_ERR_HEAD_DIM (-4)    /* head_dim other than 128 */
-#define LVX_ERR_DTYPE (-5)       /* dtype other than LVX_BF16 */
+#define LVX_ERR_DTYPE (-5)       /* dtype other than LVX_BF16 / LVX_F16 */
 #define LVX_ERR_SCALE (-6)       /* scale must be finite and > 0 */
 #define LVX_ERR_WORKSPACE (-7)   /* workspace missing or too small */
 #define LVX_ERR_UNSUPPORTED (-8) /* valid request this build does not implement */
 
 #define LVX_BF16 1
+#define LVX_F16 2               /* the reference's dtype (lv_xattn/attn.py:226,250,268) */
 
 /* Sizes shared by the attention entry points. */
 typedef struct lvx_attn_shape {
     int32_t B, Hq, Hkv, D;
     int32_t Lq;              /* text rows per sample (padded length)        */
     int32_t Lkv;             /* visual tokens per sample (padded length)    */
-    int32_t dtype;           /* LVX_BF16                                    */
+    int32_t dtype;           /* LVX_BF16 or LVX_F16: element type of q, k, v, o, dout, dq (and bf16/fp16 dk, dv) */
     float scale;             /* softmax scale, applied before the mask      */
     const int32_t* kv_len;   /* [B] valid visual tokens per sample, or NULL */
     const int32_t* kv_start; /* [B, Lq] first visible token per text row, or NULL */
@@ -80,7 +81,7 @@ const char* lvx_strerror(int code);
 
 /*
  * Flash cross-attention forward of the selected text rows against the whole
- * local K/V shard: O (bf16, normalised) and LSE.  Rows that see no key get
+ * local K/V shard: O (16-bit, normalised) and LSE.  Rows that see no key get
  * O = 0 and LSE = -inf.  Replaces the `_fwd_kernel` launch of one round
  * (lv_xattn/attn.py:140-268, launched at :390-400) and the per-round KV head
  * expansion (:271-277, :392-393), which happens in-kernel here.
@@ -119,13 +120,13 @@ int lvx_bwd_preprocess(const lvx_attn_shape* shape, const lvx_tensor* o, const l
  * (lv_xattn/flash_attn_kernels.py:364-640, 677-819; launcher :904-1020, incl.
  * the fp32 dQ scratch and `dq.copy_` of :1020) and the host-side
  * `dk += dk_delta; dv += dv_delta` of lv_xattn/attn.py:523-524.
- *   dq     : bf16, rows of the window are OVERWRITTEN (windows of different
+ *   dq     : 16-bit, rows of the window are OVERWRITTEN (windows of different
  *            rounds are disjoint, so nothing has to be accumulated);
  *   dk, dv : at Hkv heads (the group sum is taken in registers);
- *            dkv_accumulate == 0: bf16 tensors, overwritten;
+ *            dkv_accumulate == 0: 16-bit tensors, overwritten;
  *            dkv_accumulate == 1: fp32 tensors of the same indexing, added to;
  *   workspace : lvx_bwd_workspace_bytes(shape, row_count) bytes, 16-byte
- *            aligned; holds scale*dS (bf16) between the kernels of the call, the row
+ *            aligned; holds scale*dS (16-bit) between the kernels of the call, the row
  *            metadata and, for small windows, fp32 partial sums of dK/dV and dQ.
  */
 int lvx_bwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
@@ -136,15 +137,16 @@ int lvx_bwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* 
 size_t lvx_bwd_workspace_bytes(const lvx_attn_shape* shape, int32_t row_count);
 
 /*
- * dst(bf16, strided) = src(fp32, [B, H, L, D] contiguous): the final rounding of
+ * dst(dtype, strided) = src(fp32, [B, H, L, D] contiguous): the final rounding of
  * an fp32 accumulator (the `dq.copy_(dq_accum)` of flash_attn_kernels.py:1020).
  */
-int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L,
-                      int32_t D, void* stream);
+int lvx_cast_f32(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L,
+                 int32_t D, int32_t dtype, void* stream);
 
 /*
  * K/V recompute from the shared visual hidden states:
- *   K[M, N] = X[M, Dm] * W_k,   V[M, N] = X[M, Dm] * W_v      (bf16 in, fp32 accumulate)
+ *   K[M, N] = X[M, Dm] * W_k,   V[M, N] = X[M, Dm] * W_v      (16-bit in, fp32 accumulate;
+ *   `dtype`, LVX_BF16 or LVX_F16, is the element type of every matrix of the call)
  * with M = B*Lkv rows and N = Hkv*D columns, so K/V land in [B, Lkv, Hkv, D]
  * memory order.  Replaces the k_proj / v_proj nn.Linear calls inside `project`
  * (test_llama3.py:395-398) run in forward and again in backward (:197, :235).
@@ -158,14 +160,14 @@ int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_
  */
 int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw,
                 int32_t w_in_major, void* k_out, void* v_out, int64_t ldkv,
-                int32_t M, int32_t Dm, int32_t N, void* stream);
+                int32_t M, int32_t Dm, int32_t N, int32_t dtype, void* stream);
 
 /*
  * The same with the k_norm of `project` (`key_states = self.k_norm(key_states)`,
  * test_llama3.py:418; MllamaTextRMSNorm of transformers 4.47.1 over head_dim)
  * applied to K in the GEMM's epilogue, per row and per head of 128 columns:
- *   x = bf16(X W_k),  r = rsqrt(mean_d(x^2) + eps),  K = bf16(w * bf16(x * r)).
- * N must be a multiple of 128.  k_norm_w: 128 bf16 weights, 16-byte aligned.
+ *   x = rn(X W_k),  r = rsqrt(mean_d(x^2) + eps),  K = rn(w * rn(x * r)),  rn = round to dtype.
+ * N must be a multiple of 128.  k_norm_w: 128 weights of that type, 16-byte aligned.
  * Optional outputs for the norm's backward (null: not written):
  *   k_raw  : x, indexed like k_out (row stride ldkv);
  *   k_rstd : r, fp32 [M, N / 128].
@@ -173,18 +175,18 @@ int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, in
 int lvx_kv_proj_norm(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw,
                      int32_t w_in_major, void* k_out, void* v_out, int64_t ldkv,
                      int32_t M, int32_t Dm, int32_t N, const void* k_norm_w, float eps,
-                     void* k_raw, float* k_rstd, void* stream);
+                     void* k_raw, float* k_rstd, int32_t dtype, void* stream);
 
 /*
  * Backward of that norm (what autograd derives for test_llama3.py:418 when the
  * K/V gradients are propagated, which the reference's wrapper does not do,
  * :243): with xh = k_raw * r and g = dk * w, per row and head
- *   dk_raw = r * (g - xh * mean_d(g * xh)),   dw[d] += sum over rows, heads of dk * bf16(xh).
+ *   dk_raw = r * (g - xh * mean_d(g * xh)),   dw[d] += sum over rows, heads of dk * rn(xh).
  * dk_raw may alias dk.  dw: fp32 [128], ADDED to (null: not wanted).
  */
 int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk, const float* k_rstd,
                    const void* k_norm_w, void* dk_raw, int64_t lddk_raw, float* dw,
-                   int32_t M, int32_t N, void* stream);
+                   int32_t M, int32_t N, int32_t dtype, void* stream);
 
 /*
  * dX[M, Dm] = dK[M, N] * W_k^T + dV[M, N] * W_v^T  (no counterpart in the
@@ -192,7 +194,7 @@ int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk,
  */
 int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v,
                int64_t ldw, int32_t w_in_major, void* dx, int64_t lddx,
-               int32_t M, int32_t Dm, int32_t N, void* stream);
+               int32_t M, int32_t Dm, int32_t N, int32_t dtype, void* stream);
 
 /*
  * dW_k = X^T dK, dW_v = X^T dV in the layout of W (see w_in_major); the weight
@@ -200,7 +202,7 @@ int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, c
  */
 int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_t lddkv,
               void* dw_k, void* dw_v, int64_t ldw, int32_t w_in_major,
-              int32_t M, int32_t Dm, int32_t N, void* stream);
+              int32_t M, int32_t Dm, int32_t N, int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@ int check_tensor(const lvx_tensor* t) {
 
 int check_shape(const lvx_attn_shape* s) {
     if (!s) return LVX_ERR_NULL;
-    if (s->dtype != LVX_BF16) return LVX_ERR_DTYPE;
+    if (s->dtype != LVX_BF16 && s->dtype != LVX_F16) return LVX_ERR_DTYPE;
     if (s->D != 128) return LVX_ERR_HEAD_DIM;
     if (s->B <= 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Lq <= 0 || s->Lkv <= 0) return LVX_ERR_SHAPE;
     if (s->Hq % s->Hkv) return LVX_ERR_SHAPE;
@@ -70,7 +70,7 @@ const char* lvx_strerror(int code) {
         case LVX_ERR_ALIGN: return "pointer not 16-byte aligned or stride not a multiple of 8 elements";
         case LVX_ERR_SHAPE: return "bad sizes or row window";
         case LVX_ERR_HEAD_DIM: return "head_dim must be 128";
-        case LVX_ERR_DTYPE: return "dtype must be LVX_BF16";
+        case LVX_ERR_DTYPE: return "dtype must be LVX_BF16 or LVX_F16";
         case LVX_ERR_SCALE: return "scale must be finite and > 0";
         case LVX_ERR_WORKSPACE: return "workspace missing or too small";
         case LVX_ERR_UNSUPPORTED: return "not supported by this build";
@@ -101,6 +101,7 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     FwdParams p{};
+    p.f16 = s->dtype == LVX_F16;
     p.q = static_cast<const uint16_t*>(q->ptr);
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
@@ -149,6 +150,7 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     if (e != hipSuccess) return static_cast<int>(e);
 
     MergeParams m{};
+    m.f16 = s->dtype == LVX_F16;
     m.o_acc = static_cast<uint16_t*>(o->ptr);
     m.l_acc = lse;
     m.o_part = p.o;
@@ -174,6 +176,7 @@ int lvx_merge(const lvx_attn_shape* s, const lvx_tensor* o_acc, float* l_acc, co
     if (!l_acc || !l_part) return LVX_ERR_NULL;
     LVX_TRY(check_rows(s, row_begin, row_count));
     MergeParams m{};
+    m.f16 = s->dtype == LVX_F16;
     m.o_acc = static_cast<uint16_t*>(o_acc->ptr);
     m.l_acc = l_acc;
     m.o_part = static_cast<const uint16_t*>(o_part->ptr);
@@ -197,6 +200,7 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
     if (!delta) return LVX_ERR_NULL;
     LVX_TRY(check_rows(s, row_begin, row_count));
     PreParams p{};
+    p.f16 = s->dtype == LVX_F16;
     p.o = static_cast<const uint16_t*>(o->ptr);
     p.dout = static_cast<const uint16_t*>(dout->ptr);
     p.delta = delta;
@@ -312,6 +316,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     BwdParams p{};
+    p.f16 = s->dtype == LVX_F16;
     p.q = static_cast<const uint16_t*>(q->ptr);
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
@@ -382,6 +387,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
             const lvx_tensor* t = i ? dv : dk;
             // scratch memory order is [B, Lkv, Hkv, D]: cast with (H, L) = (Lkv, Hkv)
             CastParams cp{};
+            cp.f16 = p.f16;
             cp.src = scratch + i * dkv_elems;
             cp.dst = static_cast<uint16_t*>(t->ptr);
             cp.ds = Strides3{t->stride_b, t->stride_s, t->stride_h};
@@ -393,6 +399,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
 
     // dQ[b, h, rows, :] = dS^T[b, h]^T (rows x tokens) * K[b, h / G] (tokens x D), scale already in dS
     GemmParams g{};
+    g.f16 = p.f16;
     GemmProblem& pr = g.prob[0];
     pr.A[0] = p.ds_ws; pr.lda[0] = rows;
     pr.Bm[0] = p.k; pr.ldb[0] = k->stride_s;
@@ -416,6 +423,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     e = launch_gemm(g, true, true, st);
     if (e != hipSuccess) return static_cast<int>(e);
     CastParams cq{};
+    cq.f16 = p.f16;
     cq.src = dq32;
     cq.dst = static_cast<uint16_t*>(dq->ptr) + (int64_t)row_begin * dq->stride_s;
     cq.ds = st3(dq);
@@ -424,14 +432,18 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     return static_cast<int>(launch_cast(cq, st));
 }
 
-int lvx_cast_f32_bf16(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L, int32_t D,
-                      void* stream) {
+static int check_dtype(int32_t dtype) { return (dtype == LVX_BF16 || dtype == LVX_F16) ? LVX_OK : LVX_ERR_DTYPE; }
+
+int lvx_cast_f32(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, int32_t L, int32_t D,
+                 int32_t dtype, void* stream) {
+    LVX_TRY(check_dtype(dtype));
     if (!src) return LVX_ERR_NULL;
     LVX_TRY(check_tensor(dst));
     if (!aligned16(src)) return LVX_ERR_ALIGN;
     if (D != 128) return LVX_ERR_HEAD_DIM;
     if (B <= 0 || H <= 0 || L <= 0) return LVX_ERR_SHAPE;
     CastParams p{};
+    p.f16 = dtype == LVX_F16;
     p.src = src;
     p.dst = static_cast<uint16_t*>(dst->ptr);
     p.ds = st3(dst);
@@ -460,7 +472,8 @@ extern "C" {
 
 static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
                         void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N,
-                        const void* k_norm_w, float eps, void* k_raw, float* k_rstd, void* stream) {
+                        const void* k_norm_w, float eps, void* k_raw, float* k_rstd, int32_t dtype, void* stream) {
+    LVX_TRY(check_dtype(dtype));
     LVX_TRY(check_gemm_ptr(x, ldx));
     LVX_TRY(check_gemm_ptr(w_k, ldw));
     LVX_TRY(check_gemm_ptr(k_out, ldkv));
@@ -473,6 +486,7 @@ static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void*
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (ldx < Dm || ldkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
+    g.f16 = dtype == LVX_F16;
     const void* w[2] = {w_k, w_v};
     void* c[2] = {k_out, v_out};
     for (int i = 0; i < np; ++i) {
@@ -498,22 +512,23 @@ static int kv_proj_impl(const void* x, int64_t ldx, const void* w_k, const void*
 }
 
 int lvx_kv_proj(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
-                void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, void* stream) {
+                void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N, int32_t dtype, void* stream) {
     return kv_proj_impl(x, ldx, w_k, w_v, ldw, w_in_major, k_out, v_out, ldkv, M, Dm, N, nullptr, 0.f, nullptr,
-                        nullptr, stream);
+                        nullptr, dtype, stream);
 }
 
 int lvx_kv_proj_norm(const void* x, int64_t ldx, const void* w_k, const void* w_v, int64_t ldw, int32_t w_in_major,
                      void* k_out, void* v_out, int64_t ldkv, int32_t M, int32_t Dm, int32_t N,
-                     const void* k_norm_w, float eps, void* k_raw, float* k_rstd, void* stream) {
+                     const void* k_norm_w, float eps, void* k_raw, float* k_rstd, int32_t dtype, void* stream) {
     if (!k_norm_w) return LVX_ERR_NULL;
     return kv_proj_impl(x, ldx, w_k, w_v, ldw, w_in_major, k_out, v_out, ldkv, M, Dm, N, k_norm_w, eps, k_raw,
-                        k_rstd, stream);
+                        k_rstd, dtype, stream);
 }
 
 int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk, const float* k_rstd,
                    const void* k_norm_w, void* dk_raw, int64_t lddk_raw, float* dw, int32_t M, int32_t N,
-                   void* stream) {
+                   int32_t dtype, void* stream) {
+    LVX_TRY(check_dtype(dtype));
     LVX_TRY(check_gemm_ptr(dk, lddk));
     LVX_TRY(check_gemm_ptr(k_raw, ldk));
     LVX_TRY(check_gemm_ptr(dk_raw, lddk_raw));
@@ -524,6 +539,7 @@ int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk,
     if (N % 128) return LVX_ERR_HEAD_DIM;
     if (lddk < N || ldk < N || lddk_raw < N) return LVX_ERR_SHAPE;
     NormBwdParams p{};
+    p.f16 = dtype == LVX_F16;
     p.dy = static_cast<const uint16_t*>(dk);
     p.x = static_cast<const uint16_t*>(k_raw);
     p.rstd = k_rstd;
@@ -536,7 +552,9 @@ int lvx_k_norm_bwd(const void* dk, int64_t lddk, const void* k_raw, int64_t ldk,
 }
 
 int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, const void* w_v, int64_t ldw,
-               int32_t w_in_major, void* dx, int64_t lddx, int32_t M, int32_t Dm, int32_t N, void* stream) {
+               int32_t w_in_major, void* dx, int64_t lddx, int32_t M, int32_t Dm, int32_t N, int32_t dtype,
+               void* stream) {
+    LVX_TRY(check_dtype(dtype));
     LVX_TRY(check_gemm_ptr(dk, lddkv));
     LVX_TRY(check_gemm_ptr(w_k, ldw));
     LVX_TRY(check_gemm_ptr(dx, lddx));
@@ -548,6 +566,7 @@ int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, c
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (lddkv < N || lddx < Dm || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
+    g.f16 = dtype == LVX_F16;
     GemmProblem& pr = g.prob[0];
     pr.A[0] = static_cast<const uint16_t*>(dk); pr.A[1] = static_cast<const uint16_t*>(dv);
     pr.lda[0] = pr.lda[1] = lddkv;
@@ -561,7 +580,8 @@ int lvx_dx_vis(const void* dk, const void* dv, int64_t lddkv, const void* w_k, c
 }
 
 int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_t lddkv, void* dw_k, void* dw_v,
-              int64_t ldw, int32_t w_in_major, int32_t M, int32_t Dm, int32_t N, void* stream) {
+              int64_t ldw, int32_t w_in_major, int32_t M, int32_t Dm, int32_t N, int32_t dtype, void* stream) {
+    LVX_TRY(check_dtype(dtype));
     LVX_TRY(check_gemm_ptr(x, ldx));
     LVX_TRY(check_gemm_ptr(dk, lddkv));
     LVX_TRY(check_gemm_ptr(dw_k, ldw));
@@ -574,6 +594,7 @@ int lvx_dw_kv(const void* x, int64_t ldx, const void* dk, const void* dv, int64_
     if (M <= 0 || Dm <= 0 || N <= 0 || (Dm % 8) || (N % 8)) return LVX_ERR_SHAPE;
     if (ldx < Dm || lddkv < N || ldw < (w_in_major ? N : Dm)) return LVX_ERR_SHAPE;
     GemmParams g{};
+    g.f16 = dtype == LVX_F16;
     const void* d[2] = {dk, dv};
     void* c[2] = {dw_k, dw_v};
     for (int i = 0; i < np; ++i) {

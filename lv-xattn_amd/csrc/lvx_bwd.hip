@@ -68,8 +68,9 @@ constexpr int SMEM_ELEMS = LOOP_ELEMS > EPI_ELEMS ? LOOP_ELEMS : EPI_ELEMS;
 constexpr float LOG2E = 1.4426950408889634f;
 
 // BIAS: a dense fp32 bias joins the exponent, P = exp2(S*c + bias*log2e - LSE*log2e).
-template <bool MASKED, bool BIAS>
+template <bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
+    using E = Elt<F16>;
     __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
     // per-row metadata of a staged tile, one per tile buffer: 8 x 16 bytes each of
     // LSE*log2e, delta*scale, kv_start, kv_end
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) s_new[v] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) s_new = mfma32(qa[kk], breg[kk], s_new);
+            for (int kk = 0; kk < 8; ++kk) s_new = E::mfma(qa[kk], breg[kk], s_new);
         }
         if (pv_live) {
             // dO^T operands: requested once the S operands are consumed; they land while
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) pu[j][e] = pack_bf16(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
+                for (int e = 0; e < 4; ++e) pu[j][e] = E::pack(s[8 * j + 2 * e], s[8 * j + 2 * e + 1]);
             *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
             *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
 #pragma unroll
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const u32x4 a = {da[dt][j][0][0], da[dt][j][0][1], da[dt][j][1][0], da[dt][j][1][1]};
-                    acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(pu[j]), acc[dt]);
+                    acc[dt] = E::mfma(as_bf16x8(a), as_bf16x8(pu[j]), acc[dt]);
                 }
         }
         if (s_live) s_carry = s_new;
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) dp_new[v] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) dp_new = mfma32(da[kk], breg[kk], dp_new);
+            for (int kk = 0; kk < 8; ++kk) dp_new = E::mfma(da[kk], breg[kk], dp_new);
         }
         if (ds_live) {
             // Q^T operands: requested once the dO operands are consumed
@@ -365,8 +366,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                     const float d0 = (e < 2) ? da4[2 * (e & 1)] : db4[2 * (e & 1)];
                     const float d1 = (e < 2) ? da4[2 * (e & 1) + 1] : db4[2 * (e & 1) + 1];
                     // scale * P * (dP - delta), with delta * scale from the record
-                    dsu[j][e] = pack_bf16(bf16_lo(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e], p.scale, -d0),
-                                          bf16_hi(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e + 1], p.scale, -d1));
+                    dsu[j][e] = E::pack(E::lo(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e], p.scale, -d0),
+                                          E::hi(pu[j][e]) * fmaf(dp_carry[8 * j + 2 * e + 1], p.scale, -d1));
                 }
             }
             uint16_t* dsp = dst + (32 * slice + l32) * DSS + 4 * g;
@@ -380,7 +381,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const u32x4 a = {qa[dt][j][0][0], qa[dt][j][0][1], qa[dt][j][1][0], qa[dt][j][1][1]};
-                    acc[dt] = mfma32(as_bf16x8(a), as_bf16x8(dsu[j]), acc[dt]);
+                    acc[dt] = E::mfma(as_bf16x8(a), as_bf16x8(dsu[j]), acc[dt]);
                 }
         }
         if (pv_live) dp_carry = dp_new;
@@ -512,8 +513,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
                     u32x2 a;
-                    a[0] = pack_bf16(acc[dt][4 * vg], acc[dt][4 * vg + 1]);
-                    a[1] = pack_bf16(acc[dt][4 * vg + 2], acc[dt][4 * vg + 3]);
+                    a[0] = E::pack(acc[dt][4 * vg], acc[dt][4 * vg + 1]);
+                    a[1] = E::pack(acc[dt][4 * vg + 2], acc[dt][4 * vg + 3]);
                     *reinterpret_cast<u32x2*>(op + d) = a;
                 }
         }
@@ -522,15 +523,23 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
 }  // namespace
 
-hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
+namespace {
+template <bool F16>
+void launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) hipLaunchKernelGGL((bwd_kernel<true, true>), dim3(grid), dim3(NT), 0, st, p);
-        else hipLaunchKernelGGL((bwd_kernel<false, true>), dim3(grid), dim3(NT), 0, st, p);
+        if (masked) hipLaunchKernelGGL((bwd_kernel<true, true, F16>), dim3(grid), dim3(NT), 0, st, p);
+        else hipLaunchKernelGGL((bwd_kernel<false, true, F16>), dim3(grid), dim3(NT), 0, st, p);
     } else {
-        if (masked) hipLaunchKernelGGL((bwd_kernel<true, false>), dim3(grid), dim3(NT), 0, st, p);
-        else hipLaunchKernelGGL((bwd_kernel<false, false>), dim3(grid), dim3(NT), 0, st, p);
+        if (masked) hipLaunchKernelGGL((bwd_kernel<true, false, F16>), dim3(grid), dim3(NT), 0, st, p);
+        else hipLaunchKernelGGL((bwd_kernel<false, false, F16>), dim3(grid), dim3(NT), 0, st, p);
     }
+}
+}  // namespace
+
+hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
+    if (p.f16) launch_bwd_t<true>(p, masked, st);
+    else launch_bwd_t<false>(p, masked, st);
     return hipGetLastError();
 }
 

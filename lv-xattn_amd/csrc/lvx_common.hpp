@@ -50,6 +50,33 @@ __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u 
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 u) { return __builtin_bit_cast(bf16x8, u); }
 
+// The 16-bit element type of a kernel instance: packing, unpacking and the MFMA.  Operands
+// travel as bf16x8 (8 x 16 bits) whatever the type; only these functions interpret them.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+template <bool F16>
+struct Elt;
+template <>
+struct Elt<false> {   // bf16
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return pack_bf16(lo, hi); }
+    static __device__ __forceinline__ float lo(uint32_t u) { return bf16_lo(u); }
+    static __device__ __forceinline__ float hi(uint32_t u) { return bf16_hi(u); }
+    static __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32(a, b, c); }
+};
+template <>
+struct Elt<true> {    // fp16
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        f32x2 x = {lo, hi};
+        f16x2 y = __builtin_convertvector(x, f16x2);   // round-to-nearest-even
+        return __builtin_bit_cast(uint32_t, y);
+    }
+    static __device__ __forceinline__ float lo(uint32_t u) { return (float)__builtin_bit_cast(f16x2, u)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t u) { return (float)__builtin_bit_cast(f16x2, u)[1]; }
+    static __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
 // 16-byte global load, zero when !ok.
 __device__ __forceinline__ u32x4 ldg16(const void* p, bool ok) {
     u32x4 z = {0u, 0u, 0u, 0u};

@@ -44,8 +44,9 @@ constexpr float LOG2E_F = 1.4426950408889634f, LN2_F = 0.6931471805599453f;
 
 // BIAS: a dense fp32 bias is added to scale * S before the softmax; the scores are
 // then carried in log2 units (S*c + bias*log2e) instead of raw.
-template <bool MASKED, bool BIAS>
+template <bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
+    using E = Elt<F16>;
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
 
@@ -198,8 +199,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-            s0 = mfma32(ka[kk][0], qreg[kk], s0);
-            s1 = mfma32(ka[kk][1], qreg[kk], s1);
+            s0 = E::mfma(ka[kk][0], qreg[kk], s0);
+            s1 = E::mfma(ka[kk][1], qreg[kk], s1);
         }
         __builtin_amdgcn_sched_barrier(0);
         // V^T operands of this tile: requested now, they land during the softmax
@@ -273,8 +274,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
                 const float b0 = __builtin_amdgcn_exp2f(fmaf(s1[v], cc, -mc)), b1 = __builtin_amdgcn_exp2f(fmaf(s1[v + 1], cc, -mc));
                 rs0 += a0 + a1;
                 rs1 += b0 + b1;
-                u0[e] = pack_bf16(a0, a1);
-                u1[e] = pack_bf16(b0, b1);
+                u0[e] = E::pack(a0, a1);
+                u1[e] = E::pack(b0, b1);
             }
             pb[j] = as_bf16x8(u0);
             pb[2 + j] = as_bf16x8(u1);
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const u32x4 a = {va[dt][j][0][0], va[dt][j][0][1], va[dt][j][1][0], va[dt][j][1][1]};
-                acc[dt] = mfma32(as_bf16x8(a), pb[j], acc[dt]);
+                acc[dt] = E::mfma(as_bf16x8(a), pb[j], acc[dt]);
             }
     }
 
@@ -309,8 +310,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int vg = 0; vg < 4; ++vg) {
                 u32x2 w;
-                w[0] = pack_bf16(acc[dt][4 * vg] * inv, acc[dt][4 * vg + 1] * inv);
-                w[1] = pack_bf16(acc[dt][4 * vg + 2] * inv, acc[dt][4 * vg + 3] * inv);
+                w[0] = E::pack(acc[dt][4 * vg] * inv, acc[dt][4 * vg + 1] * inv);
+                w[1] = E::pack(acc[dt][4 * vg + 2] * inv, acc[dt][4 * vg + 3] * inv);
                 *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * vg + 4 * g) = w;
             }
         if (g == 0) {
@@ -322,15 +323,23 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
 }  // namespace
 
-hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
+namespace {
+template <bool F16>
+void launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) hipLaunchKernelGGL((fwd_kernel<true, true>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((fwd_kernel<false, true>), dim3(grid), dim3(256), 0, st, p);
+        if (masked) hipLaunchKernelGGL((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), 0, st, p);
     } else {
-        if (masked) hipLaunchKernelGGL((fwd_kernel<true, false>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((fwd_kernel<false, false>), dim3(grid), dim3(256), 0, st, p);
+        if (masked) hipLaunchKernelGGL((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), 0, st, p);
     }
+}
+}  // namespace
+
+hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
+    if (p.f16) launch_fwd_t<true>(p, masked, st);
+    else launch_fwd_t<false>(p, masked, st);
     return hipGetLastError();
 }
 

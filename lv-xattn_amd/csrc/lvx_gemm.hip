@@ -96,8 +96,9 @@ struct Region {
 };
 
 // GM x GN waves, each WM x WN MFMA tiles: work-group tile (32 WM GM) x (32 WN GN).
-template <bool A_MCONTIG, bool B_NCONTIG, int GM, int GN, int WM, int WN, int NS>
+template <bool A_MCONTIG, bool B_NCONTIG, int GM, int GN, int WM, int WN, int NS, bool F16>
 __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
+    using E = Elt<F16>;
     static_assert(GM * GN == 8, "8 waves");
     constexpr int TM = 32 * WM * GM, TN = 32 * WN * GN;
     using RA = Region<A_MCONTIG, TM>;
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int nt = 0; nt < WN; ++nt)
 #pragma unroll
-                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = mfma32(bn[kk][nt], am[kk][mt], acc[nt][mt]);
+                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = E::mfma(bn[kk][nt], am[kk][mt], acc[nt][mt]);
         __builtin_amdgcn_s_setprio(0);
         if (set == 0) {
             if (s + NS - 1 < steps) wait_vmcnt<(NS - 2) * LPG>();
@@ -285,7 +286,7 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
             for (int nt = 0; nt < WN; ++nt)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float x = bf16_hi(pack_bf16(0.f, acc[nt][mt][i]));   // the product as bf16
+                    const float x = E::hi(E::pack(0.f, acc[nt][mt][i]));   // the product as bf16
                     acc[nt][mt][i] = x;
                     ss = fmaf(x, x, ss);
                 }
@@ -316,15 +317,15 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
                         const float a[4] = {acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1], acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]};
                         if (p.c_raw) {
                             u32x2 w;
-                            w[0] = pack_bf16(a[0], a[1]);
-                            w[1] = pack_bf16(a[2], a[3]);
+                            w[0] = E::pack(a[0], a[1]);
+                            w[1] = E::pack(a[2], a[3]);
                             *reinterpret_cast<u32x2*>(p.c_raw + (Cz - pr.C) + (int64_t)m * pr.ldc + n) = w;
                         }
                         const u32x2 wt = *reinterpret_cast<const u32x2*>(p.norm_w + (n & 127));
-                        const u32x2 h = {pack_bf16(a[0] * r, a[1] * r), pack_bf16(a[2] * r, a[3] * r)};
+                        const u32x2 h = {E::pack(a[0] * r, a[1] * r), E::pack(a[2] * r, a[3] * r)};
                         u32x2 y;
-                        y[0] = pack_bf16(bf16_lo(wt[0]) * bf16_lo(h[0]), bf16_hi(wt[0]) * bf16_hi(h[0]));
-                        y[1] = pack_bf16(bf16_lo(wt[1]) * bf16_lo(h[1]), bf16_hi(wt[1]) * bf16_hi(h[1]));
+                        y[0] = E::pack(E::lo(wt[0]) * E::lo(h[0]), E::hi(wt[0]) * E::hi(h[0]));
+                        y[1] = E::pack(E::lo(wt[1]) * E::lo(h[1]), E::hi(wt[1]) * E::hi(h[1]));
                         *reinterpret_cast<u32x2*>(Cz + (int64_t)m * pr.ldc + n) = y;
                     }
                 }
@@ -342,12 +343,24 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
                 const int n = n0 + 32 * (WN * wn + nt) + 8 * vg + 4 * g;
                 if (n < p.N) {
                     u32x2 w;
-                    w[0] = pack_bf16(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
-                    w[1] = pack_bf16(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
+                    w[0] = E::pack(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
+                    w[1] = E::pack(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
                     *reinterpret_cast<u32x2*>(Cz + (int64_t)m * pr.ldc + n) = w;
                 }
             }
     }
+}
+
+template <int GM, int GN, int WM, int WN, int NS, bool F16>
+void launch_cfg_t(const GemmParams& p, int grid, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+    if (!a_mcontig && !b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<false, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+    else if (!a_mcontig && b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<false, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+    else if (a_mcontig && !b_ncontig)
+        hipLaunchKernelGGL((gemm_kernel<true, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+    else
+        hipLaunchKernelGGL((gemm_kernel<true, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
 }
 
 template <int GM, int GN, int WM, int WN, int NS>
@@ -357,14 +370,8 @@ hipError_t launch_cfg(GemmParams p, bool a_mcontig, bool b_ncontig, hipStream_t 
     p.tiles_n = (p.N + TN - 1) / TN;
     p.total_wg = p.nprob * p.nbatch * p.tiles_m * p.tiles_n * (p.k_splits > 1 ? p.k_splits : 1);
     const int grid = ((p.total_wg + 7) / 8) * 8;
-    if (!a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, false, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
-    else if (!a_mcontig && b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, true, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
-    else if (a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<true, false, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
-    else
-        hipLaunchKernelGGL((gemm_kernel<true, true, GM, GN, WM, WN, NS>), dim3(grid), dim3(512), 0, st, p);
+    if (p.f16) launch_cfg_t<GM, GN, WM, WN, NS, true>(p, grid, a_mcontig, b_ncontig, st);
+    else launch_cfg_t<GM, GN, WM, WN, NS, false>(p, grid, a_mcontig, b_ncontig, st);
     return hipGetLastError();
 }
 

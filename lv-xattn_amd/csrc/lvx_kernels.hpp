@@ -32,6 +32,7 @@ struct FwdParams {
     int row_begin, row_end;
     int n_row_tiles, n_head_groups, nsplit, split_len, total_wg;
     float scale, scale_log2e;
+    int f16;                   // element type of q, k, v, o: 0 bf16, 1 fp16
 };
 
 struct MergeParams {
@@ -46,6 +47,7 @@ struct MergeParams {
     int nparts;
     int use_acc;               // 1: fold into the existing accumulator, 0: overwrite
     int B, Hq, Lq, row_begin, row_end;
+    int f16;
 };
 
 struct PreParams {
@@ -54,6 +56,7 @@ struct PreParams {
     float* delta;
     Strides3 os, ds;
     int B, Hq, Lq, row_begin, row_end;
+    int f16;
 };
 
 struct BwdParams {
@@ -84,6 +87,7 @@ struct BwdParams {
     // its tokens) as up to 4 runs of consecutive tiles, live_runs[(b * n_kv_blocks + block) * 8
     // + 2 i + {0, 1}] = first tile and number of tiles of run i (0 tiles: unused).  Null: every tile.
     const int32_t* live_runs;
+    int f16;                   // element type of q, k, v, dout, the dS^T workspace and (mode 0) dk, dv
 };
 
 // Which (token block, 32-row tile) pairs an interval mask leaves alive, at the granularity the
@@ -127,6 +131,7 @@ struct CastParams {
     Strides3 ds;
     int B, H, L;
     int transposed;   // 0: src is [B*H][L][D]; 1: src is [B*H][D][L]
+    int f16;          // destination type: 0 bf16, 1 fp16
 };
 
 // One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].
@@ -166,6 +171,7 @@ struct GemmParams {
     // Per (outer batch index, M tile) contraction range of segment 0: k_range[(zo * tiles_m +
     // tm) * 2 + {0, 1}] = first and one-past-last k (multiples of 128); null: all of K[0].
     const int32_t* k_range;
+    int f16;                   // element type of A, B, C (and the norm weight): 0 bf16, 1 fp16
     // Split contraction (single-segment problems): k_splits work-groups per C tile, each
     // contracting k_split_len values of k (a multiple of 128) and adding its partial tile
     // with fp32 atomics to the TRANSPOSED scratch c32[z * c32_batch + n * c32_ld + m] (zeroed
@@ -198,6 +204,7 @@ struct NormBwdParams {
     float* dw;        // [128] fp32, added to (null: not wanted)
     int64_t ldy, ldx, lddx;
     int M, heads;
+    int f16;
 };
 hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st);
 // a_mcontig: A is stored [K][M] (m contiguous); b_ncontig: B is stored [K][N].

@@ -16,16 +16,19 @@ namespace {
 constexpr int D = 128;
 constexpr int MAX_PARTS = 16;
 
+template <class E>
 __device__ __forceinline__ void unpack8(u32x4 u, float f[8]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        f[2 * j] = bf16_lo(u[j]);
-        f[2 * j + 1] = bf16_hi(u[j]);
+        f[2 * j] = E::lo(u[j]);
+        f[2 * j + 1] = E::hi(u[j]);
     }
 }
 
 // (o_acc, l_acc) <- merge(acc?, part_0 .. part_{n-1}) for every (b, h, row).
+template <bool F16>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
+    using E = Elt<F16>;
     const int nrows = p.row_end - p.row_begin;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     uint16_t* oa = p.o_acc + b * p.oa.b + h * p.oa.h + (int64_t)row * p.oa.s + chunk * 8;
     if (p.use_acc) {
         float f[8];
-        unpack8(*reinterpret_cast<const u32x4*>(oa), f);
+        unpack8<E>(*reinterpret_cast<const u32x4*>(oa), f);
         const float w = wa * inv;
 #pragma unroll
         for (int j = 0; j < 8; ++j) out[j] = f[j] * w;
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     for (int i = 0; i < MAX_PARTS; ++i) {
         if (i < p.nparts) {
             float f[8];
-            unpack8(*reinterpret_cast<const u32x4*>(op + i * p.o_part_stride), f);
+            unpack8<E>(*reinterpret_cast<const u32x4*>(op + i * p.o_part_stride), f);
             const float w = lp[i] * inv;
             // a part with weight 0 may hold anything (it saw no key)
             if (w > 0.f) {
@@ -85,12 +88,14 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     }
     u32x4 u;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) u[j] = pack_bf16(out[2 * j], out[2 * j + 1]);
+    for (int j = 0; j < 4; ++j) u[j] = E::pack(out[2 * j], out[2 * j + 1]);
     *reinterpret_cast<u32x4*>(oa) = u;
     if (chunk == 0) p.l_acc[(int64_t)bh * p.l_acc_bh + row] = den > 0.f ? ms + __logf(den) : -INFINITY;
 }
 
+template <bool F16>
 __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
+    using E = Elt<F16>;
     const int nrows = p.row_end - p.row_begin;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
@@ -101,8 +106,8 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
     const int bh = (int)(rr / nrows);
     const int b = bh / p.Hq, h = bh % p.Hq;
     float fo[8], fd[8];
-    unpack8(ldg16(p.o + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s + chunk * 8, ok), fo);
-    unpack8(ldg16(p.dout + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8, ok), fd);
+    unpack8<E>(ldg16(p.o + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s + chunk * 8, ok), fo);
+    unpack8<E>(ldg16(p.dout + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8, ok), fd);
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
@@ -187,7 +192,9 @@ __global__ __launch_bounds__(64) void bwd_live_kernel(const LiveParams p) {
     for (int i = nr; i < 4; ++i) { out[2 * i] = 0; out[2 * i + 1] = 0; }
 }
 
+template <bool F16>
 __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
+    using E = Elt<F16>;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
     const int64_t r = idx >> 4;
@@ -198,16 +205,18 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     const f32x4* s = reinterpret_cast<const f32x4*>(p.src + r * D + chunk * 8);
     const f32x4 a = s[0], c = s[1];
     u32x4 u;
-    u[0] = pack_bf16(a[0], a[1]);
-    u[1] = pack_bf16(a[2], a[3]);
-    u[2] = pack_bf16(c[0], c[1]);
-    u[3] = pack_bf16(c[2], c[3]);
+    u[0] = E::pack(a[0], a[1]);
+    u[1] = E::pack(a[2], a[3]);
+    u[2] = E::pack(c[0], c[1]);
+    u[3] = E::pack(c[2], c[3]);
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
 // Same from a transposed source [B*H][D][L]: adjacent threads take adjacent rows, so the
 // eight strided reads of a thread are coalesced across the wave.
+template <bool F16>
 __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
+    using E = Elt<F16>;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (int64_t)p.B * p.H * p.L * 16) return;
     const int row = (int)(idx % p.L);
@@ -220,7 +229,7 @@ __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
     for (int j = 0; j < 8; ++j) a[j] = s[(int64_t)j * p.L];
     u32x4 u;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) u[j] = pack_bf16(a[2 * j], a[2 * j + 1]);
+    for (int j = 0; j < 4; ++j) u[j] = E::pack(a[2 * j], a[2 * j + 1]);
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
@@ -228,14 +237,16 @@ __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
 //   dx = r * (gg - xh * mean(gg * xh)),   dw += sum over rows of dy * bf16(xh).
 // 16 lanes per row (8 columns each); a thread keeps the dw partial sums of its 8 columns
 // over the rows it visits, the block folds them through LDS and adds them with atomics.
+template <bool F16>
 __global__ __launch_bounds__(256) void norm_bwd_kernel(const NormBwdParams p) {
+    using E = Elt<F16>;
     __shared__ float fold[16][16][8];
     const int sub = threadIdx.x & 15, grp = threadIdx.x >> 4;
     const int64_t nrows = (int64_t)p.M * p.heads;
     const u32x4 wu = *reinterpret_cast<const u32x4*>(p.w + sub * 8);
     float w[8], dwp[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { w[2 * j] = bf16_lo(wu[j]); w[2 * j + 1] = bf16_hi(wu[j]); }
+    for (int j = 0; j < 4; ++j) { w[2 * j] = E::lo(wu[j]); w[2 * j + 1] = E::hi(wu[j]); }
 #pragma unroll
     for (int j = 0; j < 8; ++j) dwp[j] = 0.f;
     for (int64_t row = (int64_t)blockIdx.x * 16 + grp; row < nrows; row += (int64_t)gridDim.x * 16) {
@@ -247,14 +258,14 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const NormBwdParams p) {
         float gg[8], xh[8], c = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float d0 = bf16_lo(du[j]), d1 = bf16_hi(du[j]);
-            xh[2 * j] = bf16_lo(xu[j]) * r;
-            xh[2 * j + 1] = bf16_hi(xu[j]) * r;
+            const float d0 = E::lo(du[j]), d1 = E::hi(du[j]);
+            xh[2 * j] = E::lo(xu[j]) * r;
+            xh[2 * j + 1] = E::hi(xu[j]) * r;
             gg[2 * j] = d0 * w[2 * j];
             gg[2 * j + 1] = d1 * w[2 * j + 1];
-            const uint32_t xb = pack_bf16(xh[2 * j], xh[2 * j + 1]);
-            dwp[2 * j] = fmaf(d0, bf16_lo(xb), dwp[2 * j]);
-            dwp[2 * j + 1] = fmaf(d1, bf16_hi(xb), dwp[2 * j + 1]);
+            const uint32_t xb = E::pack(xh[2 * j], xh[2 * j + 1]);
+            dwp[2 * j] = fmaf(d0, E::lo(xb), dwp[2 * j]);
+            dwp[2 * j + 1] = fmaf(d1, E::hi(xb), dwp[2 * j + 1]);
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) c = fmaf(gg[j], xh[j], c);
@@ -264,7 +275,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const NormBwdParams p) {
         u32x4 out;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            out[j] = pack_bf16(r * (gg[2 * j] - xh[2 * j] * c), r * (gg[2 * j + 1] - xh[2 * j + 1] * c));
+            out[j] = E::pack(r * (gg[2 * j] - xh[2 * j] * c), r * (gg[2 * j + 1] - xh[2 * j + 1] * c));
         *reinterpret_cast<u32x4*>(p.dx + m * p.lddx + h * 128 + sub * 8) = out;
     }
     if (!p.dw) return;
@@ -294,14 +305,16 @@ inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(merge_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    if (p.f16) hipLaunchKernelGGL(merge_kernel<true>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(merge_kernel<false>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(preprocess_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    if (p.f16) hipLaunchKernelGGL(preprocess_kernel<true>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(preprocess_kernel<false>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
@@ -336,17 +349,22 @@ hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.M * p.heads;
     if (rows == 0) return hipSuccess;
     const int grid = (int)std::min<int64_t>((rows + 15) / 16, 2048);
-    hipLaunchKernelGGL(norm_bwd_kernel, dim3(grid), dim3(256), 0, st, p);
+    if (p.f16) hipLaunchKernelGGL(norm_bwd_kernel<true>, dim3(grid), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(norm_bwd_kernel<false>, dim3(grid), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
 hipError_t launch_cast(const CastParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.H * p.L;
     if (rows == 0) return hipSuccess;
-    if (p.transposed)
-        hipLaunchKernelGGL(cast_t_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
-    else
-        hipLaunchKernelGGL(cast_kernel, dim3(blocks_for(rows)), dim3(256), 0, st, p);
+    const dim3 grid(blocks_for(rows));
+    if (p.transposed) {
+        if (p.f16) hipLaunchKernelGGL(cast_t_kernel<true>, grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(cast_t_kernel<false>, grid, dim3(256), 0, st, p);
+    } else {
+        if (p.f16) hipLaunchKernelGGL(cast_kernel<true>, grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(cast_kernel<false>, grid, dim3(256), 0, st, p);
+    }
     return hipGetLastError();
 }
 

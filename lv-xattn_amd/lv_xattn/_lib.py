@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LVX_LIB") or os.path.join(_HERE, "liblvx.so")
 
 LVX_BF16 = 1
+LVX_F16 = 2
 
 
 class LvxError(RuntimeError):
@@ -48,17 +49,17 @@ SYMBOLS = {
     "lvx_bwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, _P, _T, _T, _T, C.c_int32, C.c_int32, C.c_int32,
                           _P, C.c_size_t, _P]),
     "lvx_bwd_workspace_bytes": (C.c_size_t, [_SHAPE, C.c_int32]),
-    "lvx_cast_f32_bf16": (C.c_int, [_P, _T, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
+    "lvx_cast_f32": (C.c_int, [_P, _T, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_kv_proj": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, _P, C.c_int64,
-                              C.c_int32, C.c_int32, C.c_int32, _P]),
+                              C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_kv_proj_norm": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, _P, C.c_int64,
-                                   C.c_int32, C.c_int32, C.c_int32, _P, C.c_float, _P, _P, _P]),
+                                   C.c_int32, C.c_int32, C.c_int32, _P, C.c_float, _P, _P, C.c_int32, _P]),
     "lvx_k_norm_bwd": (C.c_int, [_P, C.c_int64, _P, C.c_int64, _P, _P, _P, C.c_int64, _P,
-                                 C.c_int32, C.c_int32, _P]),
+                                 C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_dx_vis": (C.c_int, [_P, _P, C.c_int64, _P, _P, C.c_int64, C.c_int32, _P, C.c_int64,
-                             C.c_int32, C.c_int32, C.c_int32, _P]),
+                             C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_dw_kv": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, _P, _P, C.c_int64, C.c_int32,
-                            C.c_int32, C.c_int32, C.c_int32, _P]),
+                            C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P]),
 }
 
 _lib: Optional[C.CDLL] = None

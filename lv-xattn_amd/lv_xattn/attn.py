@@ -184,6 +184,6 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
             ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
                     accumulate_dkv=True, workspace=ws, bias=bias)
         # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
-        ops.cast_f32_bf16(dk_acc.transpose(1, 2), dk.transpose(1, 2))
-        ops.cast_f32_bf16(dv_acc.transpose(1, 2), dv.transpose(1, 2))
+        ops.cast_f32(dk_acc.transpose(1, 2), dk.transpose(1, 2))
+        ops.cast_f32(dv_acc.transpose(1, 2), dv.transpose(1, 2))
     return dq, dk, dv

@@ -77,9 +77,9 @@ def lv_xattn_attention_forward(module, query, key, value, attention_mask: Option
 
 
 def _require_supported(query, key, dropout):
-    if not (query.is_cuda and query.dtype == torch.bfloat16 and query.shape[-1] == 128 and dropout == 0.0
+    if not (query.is_cuda and query.dtype in (torch.bfloat16, torch.float16) and query.shape[-1] == 128 and dropout == 0.0
             and query.shape[1] % key.shape[1] == 0):
-        raise LvxError("lv_xattn cross-attention needs bf16 tensors on the GPU, head_dim 128, no dropout and "
+        raise LvxError("lv_xattn cross-attention needs bf16 or fp16 tensors on the GPU, head_dim 128, no dropout and "
                        f"Hkv | Hq; got {query.dtype} on {query.device}, q {tuple(query.shape)}, "
                        f"k {tuple(key.shape)}, dropout {dropout}")
 
@@ -100,9 +100,9 @@ def _recompute_forward(self, hidden_states, cross_attention_states=None, past_ke
                                        attention_mask, use_cache, **kwargs)
     bsz, q_len, _ = hidden_states.size()
     dropout = self.dropout if self.training else 0.0
-    if not (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and self.head_dim == 128
+    if not (hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float16) and self.head_dim == 128
             and dropout == 0.0):
-        raise LvxError("lv_xattn cross-attention needs bf16 tensors on the GPU, head_dim 128 and no dropout")
+        raise LvxError("lv_xattn cross-attention needs bf16 or fp16 tensors on the GPU, head_dim 128 and no dropout")
     key = (self._lvx_rounds, self._lvx_batched, self._lvx_weight_grads)
     if key not in _recompute:
         _recompute[key] = create_attention_class("lv_xattn", rounds=key[0], batched=key[1],

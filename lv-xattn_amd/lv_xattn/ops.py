@@ -33,15 +33,25 @@ class Mask:
         return Mask(f(self.kv_len), f(self.kv_start), f(self.kv_end))
 
 
+_DTYPES = {torch.bfloat16: _lib.LVX_BF16, torch.float16: _lib.LVX_F16}
+
+
+def dtype_code(t: torch.Tensor, *others: torch.Tensor) -> int:
+    """LVX_BF16 / LVX_F16 for the element type all the given tensors share."""
+    if t.dtype not in _DTYPES or any(o.dtype != t.dtype for o in others):
+        raise LvxError("bf16 or fp16 tensors of one type required, got "
+                       + " / ".join(str(x.dtype) for x in (t,) + others))
+    return _DTYPES[t.dtype]
+
+
 def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask],
            bias: Optional[torch.Tensor] = None) -> AttnShape:
-    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16:
-        raise LvxError(f"bf16 tensors required, got {q.dtype} / {k.dtype}")
+    dt = dtype_code(q, k)
     B, Hq, Lq, D = q.shape
     Bk, Hkv, Lkv, Dk = k.shape
     if B != Bk or D != Dk:
         raise LvxError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
-    s = AttnShape(B, Hq, Hkv, D, Lq, Lkv, _lib.LVX_BF16, float(scale), None, None, None)
+    s = AttnShape(B, Hq, Hkv, D, Lq, Lkv, dt, float(scale), None, None, None)
     if mask is not None:
         for name in ("kv_len", "kv_start", "kv_end"):
             t = getattr(mask, name)
@@ -87,7 +97,7 @@ def fwd(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask
 def merge(o_acc, l_acc, o_part, l_part, row_begin=0, row_count=None) -> None:
     """(o_acc, l_acc) <- LSE-merge of itself with (o_part, l_part), in place."""
     B, Hq, Lq, D = o_acc.shape
-    s = AttnShape(B, Hq, Hq, D, Lq, 1, _lib.LVX_BF16, 1.0, None, None, None)
+    s = AttnShape(B, Hq, Hq, D, Lq, 1, dtype_code(o_acc, o_part), 1.0, None, None, None)
     if row_count is None:
         row_count = Lq - row_begin
     _check_lse(l_acc, o_acc)
@@ -99,7 +109,7 @@ def merge(o_acc, l_acc, o_part, l_part, row_begin=0, row_count=None) -> None:
 
 def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
     B, Hq, Lq, D = o.shape
-    s = AttnShape(B, Hq, Hq, D, Lq, 1, _lib.LVX_BF16, 1.0, None, None, None)
+    s = AttnShape(B, Hq, Hq, D, Lq, 1, dtype_code(o, dout), 1.0, None, None, None)
     if row_count is None:
         row_count = Lq - row_begin
     _check_lse(delta, o)
@@ -127,9 +137,9 @@ def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=Non
         row_count = q.shape[2] - row_begin
     _check_lse(lse, q)
     _check_lse(delta, q)
-    if dq.dtype != torch.bfloat16 or dq.shape != q.shape:
-        raise LvxError("dq must be a bf16 tensor shaped like q")
-    want = torch.float32 if accumulate_dkv else torch.bfloat16
+    if dq.dtype != q.dtype or dq.shape != q.shape:
+        raise LvxError("dq must be a tensor of q's type and shape")
+    want = torch.float32 if accumulate_dkv else q.dtype
     if dk.dtype != want or dv.dtype != want or dk.shape != k.shape or dv.shape != k.shape:
         raise LvxError(f"dk/dv must be {want} tensors shaped like k")
     if workspace is None:
@@ -141,19 +151,19 @@ def bwd(q, k, v, dout, lse, delta, dq, dk, dv, scale, row_begin=0, row_count=Non
     check(rc, "lvx_bwd")
 
 
-def cast_f32_bf16(src: torch.Tensor, dst: torch.Tensor) -> None:
-    """dst (bf16, [B,H,L,D] any strides) = src (fp32, memory order [B,H,L,D])."""
+def cast_f32(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst (bf16 or fp16, [B,H,L,D] any strides) = src (fp32, memory order [B,H,L,D])."""
     B, H, L, D = dst.shape
-    if src.dtype != torch.float32 or src.numel() != dst.numel() or dst.dtype != torch.bfloat16:
-        raise LvxError("cast_f32_bf16: fp32 source and bf16 destination of equal size required")
-    rc = load().lvx_cast_f32_bf16(src.data_ptr(), C.byref(t4(dst)), B, H, L, D, stream_ptr())
-    check(rc, "lvx_cast_f32_bf16")
+    if src.dtype != torch.float32 or src.numel() != dst.numel():
+        raise LvxError("cast_f32: fp32 source and 16-bit destination of equal size required")
+    rc = load().lvx_cast_f32(src.data_ptr(), C.byref(t4(dst)), B, H, L, D, dtype_code(dst), stream_ptr())
+    check(rc, "lvx_cast_f32")
 
 
 def _rows2d(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
     """[..., C] tensor whose leading dims collapse to rows with one stride."""
-    if t.dtype != torch.bfloat16:
-        raise LvxError(f"{name}: bf16 required")
+    if t.dtype not in _DTYPES:
+        raise LvxError(f"{name}: bf16 or fp16 required")
     t2 = t.reshape(-1, t.shape[-1]) if t.is_contiguous() else None
     if t2 is None:
         raise LvxError(f"{name}: contiguous tensor required")
@@ -178,7 +188,8 @@ def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True,
     if ldw != ldw2 or w_k.shape != w_v.shape:
         raise LvxError("w_k and w_v must have the same shape")
     D = N // n_kv_heads
-    k = torch.empty(B, Lkv, N, dtype=torch.bfloat16, device=x_vis.device)
+    dt = dtype_code(x_vis, w_k, w_v)
+    k = torch.empty(B, Lkv, N, dtype=x_vis.dtype, device=x_vis.device)
     v = torch.empty_like(k)
 
     def heads(t):
@@ -188,27 +199,27 @@ def kv_proj(x_vis, w_k, w_v, n_kv_heads: int, w_in_major: bool = True,
         if for_backward:
             raise LvxError("for_backward only applies with k_norm_weight")
         rc = load().lvx_kv_proj(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
-                                M, Dm, N, stream_ptr())
+                                M, Dm, N, dt, stream_ptr())
         check(rc, "lvx_kv_proj")
         return heads(k), heads(v)
-    wn = _norm_weight(k_norm_weight, D, x_vis.device)
+    wn = _norm_weight(k_norm_weight, D, x_vis)
     k_raw = torch.empty_like(k) if for_backward else None
     rstd = torch.empty(B, Lkv, n_kv_heads, dtype=torch.float32, device=x_vis.device) if for_backward else None
     rc = load().lvx_kv_proj_norm(xp, ldx, wkp, wvp, ldw, 1 if w_in_major else 0, k.data_ptr(), v.data_ptr(), N,
                                  M, Dm, N, wn.data_ptr(), float(eps),
                                  k_raw.data_ptr() if for_backward else None,
-                                 rstd.data_ptr() if for_backward else None, stream_ptr())
+                                 rstd.data_ptr() if for_backward else None, dt, stream_ptr())
     check(rc, "lvx_kv_proj_norm")
     if for_backward:
         return heads(k), heads(v), heads(k_raw), rstd
     return heads(k), heads(v)
 
 
-def _norm_weight(w: torch.Tensor, D: int, dev) -> torch.Tensor:
-    if w.dtype != torch.bfloat16 or tuple(w.shape) != (D,) or D != 128:
-        raise LvxError(f"k_norm_weight must be bf16 [128], got {w.dtype} {tuple(w.shape)}")
+def _norm_weight(w: torch.Tensor, D: int, like: torch.Tensor) -> torch.Tensor:
+    if w.dtype != like.dtype or tuple(w.shape) != (D,) or D != 128:
+        raise LvxError(f"the norm weight must be {like.dtype} [128], got {w.dtype} {tuple(w.shape)}")
     w = w.detach()
-    if w.device != dev:
+    if w.device != like.device:
         raise LvxError("k_norm_weight is on another device")
     if not w.is_contiguous() or w.data_ptr() % 16:
         w = w.contiguous().clone()
@@ -222,13 +233,14 @@ def k_norm_bwd(dk, k_raw, k_rstd, k_norm_weight, want_dw: bool = True):
     B, Hkv, Lkv, D = dk.shape
     dk2, kr2 = _token_major(dk, "dk"), _token_major(k_raw, "k_raw")
     N = Hkv * D
-    wn = _norm_weight(k_norm_weight, D, dk.device)
+    wn = _norm_weight(k_norm_weight, D, dk)
     if k_rstd.dtype != torch.float32 or k_rstd.numel() != B * Lkv * Hkv or not k_rstd.is_contiguous():
         raise LvxError("k_rstd must be contiguous fp32 [B, Lkv, Hkv]")
-    out = torch.empty(B, Lkv, N, dtype=torch.bfloat16, device=dk.device)
+    out = torch.empty(B, Lkv, N, dtype=dk.dtype, device=dk.device)
     dw = torch.zeros(D, dtype=torch.float32, device=dk.device) if want_dw else None
     rc = load().lvx_k_norm_bwd(dk2.data_ptr(), N, kr2.data_ptr(), N, k_rstd.data_ptr(), wn.data_ptr(),
-                               out.data_ptr(), N, dw.data_ptr() if want_dw else None, B * Lkv, N, stream_ptr())
+                               out.data_ptr(), N, dw.data_ptr() if want_dw else None, B * Lkv, N,
+                               dtype_code(dk, k_raw), stream_ptr())
     check(rc, "lvx_k_norm_bwd")
     return out.view(B, Lkv, Hkv, D).transpose(1, 2), dw
 
@@ -243,7 +255,8 @@ def q_proj(x, w_q, n_heads: int, w_in_major: bool = True, q_norm_weight: Optiona
     xp, M, ldx = _rows2d(x, "x")
     wp, _, ldw = _rows2d(w_q, "w_q")
     D = N // n_heads
-    q = torch.empty(B, Lq, N, dtype=torch.bfloat16, device=x.device)
+    dt = dtype_code(x, w_q)
+    q = torch.empty(B, Lq, N, dtype=x.dtype, device=x.device)
 
     def heads(t):
         return t.view(B, Lq, n_heads, D).transpose(1, 2)
@@ -252,16 +265,16 @@ def q_proj(x, w_q, n_heads: int, w_in_major: bool = True, q_norm_weight: Optiona
         if for_backward:
             raise LvxError("for_backward only applies with q_norm_weight")
         rc = load().lvx_kv_proj(xp, ldx, wp, None, ldw, 1 if w_in_major else 0, q.data_ptr(), None, N,
-                                M, Dm, N, stream_ptr())
+                                M, Dm, N, dt, stream_ptr())
         check(rc, "lvx_kv_proj")
         return heads(q)
-    wn = _norm_weight(q_norm_weight, D, x.device)
+    wn = _norm_weight(q_norm_weight, D, x)
     raw = torch.empty_like(q) if for_backward else None
     rstd = torch.empty(B, Lq, n_heads, dtype=torch.float32, device=x.device) if for_backward else None
     rc = load().lvx_kv_proj_norm(xp, ldx, wp, None, ldw, 1 if w_in_major else 0, q.data_ptr(), None, N,
                                  M, Dm, N, wn.data_ptr(), float(eps),
                                  raw.data_ptr() if for_backward else None,
-                                 rstd.data_ptr() if for_backward else None, stream_ptr())
+                                 rstd.data_ptr() if for_backward else None, dt, stream_ptr())
     check(rc, "lvx_kv_proj_norm")
     if for_backward:
         return heads(q), heads(raw), rstd
@@ -277,16 +290,17 @@ def q_proj_bwd(x, dq_raw, w_q, w_in_major: bool = True, want_dw: bool = True):
     Dm = w_q.shape[0] if w_in_major else w_q.shape[1]
     wp, _, ldw = _rows2d(w_q, "w_q")
     xp, M, ldx = _rows2d(x, "x")
-    dx = torch.empty(B, Lq, Dm, dtype=torch.bfloat16, device=x.device)
+    dt = dtype_code(x, dq_raw, w_q)
+    dx = torch.empty(B, Lq, Dm, dtype=x.dtype, device=x.device)
     rc = load().lvx_dx_vis(d2.data_ptr(), None, N, wp, None, ldw, 1 if w_in_major else 0, dx.data_ptr(), Dm,
-                           M, Dm, N, stream_ptr())
+                           M, Dm, N, dt, stream_ptr())
     check(rc, "lvx_dx_vis")
     dw = None
     if want_dw:
         shape = (Dm, N) if w_in_major else (N, Dm)
-        dw = torch.empty(*shape, dtype=torch.bfloat16, device=x.device)
+        dw = torch.empty(*shape, dtype=x.dtype, device=x.device)
         rc = load().lvx_dw_kv(xp, ldx, d2.data_ptr(), None, N, dw.data_ptr(), None, shape[1],
-                              1 if w_in_major else 0, M, Dm, N, stream_ptr())
+                              1 if w_in_major else 0, M, Dm, N, dt, stream_ptr())
         check(rc, "lvx_dw_kv")
     return dx, dw
 
@@ -307,9 +321,9 @@ def dx_vis(dk, dv, w_k, w_v, w_in_major: bool = True) -> torch.Tensor:
     Dm = w_k.shape[0] if w_in_major else w_k.shape[1]
     wkp, _, ldw = _rows2d(w_k, "w_k")
     wvp, _, _ = _rows2d(w_v, "w_v")
-    dx = torch.empty(B, Lkv, Dm, dtype=torch.bfloat16, device=dk.device)
+    dx = torch.empty(B, Lkv, Dm, dtype=dk.dtype, device=dk.device)
     rc = load().lvx_dx_vis(dk2.data_ptr(), dv2.data_ptr(), N, wkp, wvp, ldw, 1 if w_in_major else 0,
-                           dx.data_ptr(), Dm, B * Lkv, Dm, N, stream_ptr())
+                           dx.data_ptr(), Dm, B * Lkv, Dm, N, dtype_code(dk, dv, w_k, w_v), stream_ptr())
     check(rc, "lvx_dx_vis")
     return dx
 
@@ -322,10 +336,10 @@ def dw_kv(x_vis, dk, dv, w_in_major: bool = True):
     dk2, dv2 = _token_major(dk, "dk"), _token_major(dv, "dv")
     xp, M, ldx = _rows2d(x_vis, "x_vis")
     shape = (Dm, N) if w_in_major else (N, Dm)
-    dwk = torch.empty(*shape, dtype=torch.bfloat16, device=x_vis.device)
+    dwk = torch.empty(*shape, dtype=x_vis.dtype, device=x_vis.device)
     dwv = torch.empty_like(dwk)
     rc = load().lvx_dw_kv(xp, ldx, dk2.data_ptr(), dv2.data_ptr(), N, dwk.data_ptr(), dwv.data_ptr(), shape[1],
-                          1 if w_in_major else 0, M, Dm, N, stream_ptr())
+                          1 if w_in_major else 0, M, Dm, N, dtype_code(x_vis, dk, dv), stream_ptr())
     check(rc, "lvx_dw_kv")
     return dwk, dwv
 

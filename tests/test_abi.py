@@ -64,7 +64,7 @@ def _fwd(lib, shape, q=None, k=None, v=None, o=None, lse=0x2000, rb=0, rc=64, sp
 
 def test_forward_rejects_bad_arguments_before_launch(lib):
     assert _fwd(lib, _shape(D=64)) == -4
-    assert _fwd(lib, _shape(dtype=2)) == -5
+    assert _fwd(lib, _shape(dtype=3)) == -5            # 1 = bf16, 2 = fp16
     assert _fwd(lib, _shape(Hq=7)) == -3
     assert _fwd(lib, _shape(scale=0.0)) == -6
     assert _fwd(lib, _shape(scale=float("nan"))) == -6
@@ -108,21 +108,24 @@ def test_other_entry_points_reject_bad_arguments(lib):
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need - 1, None) == -7
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, None, 0, None) == -7
-    assert lib.lvx_cast_f32_bf16(0x1000, C.byref(t), 1, 8, 64, 64, None) == -4
-    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, None) == -3
-    assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, None) == -1
-    assert lib.lvx_dx_vis(0x1000, 0x1100, 256, 0x2000, 0x3000, 250, 1, 0x4000, 512, 100, 512, 256, None) == -2
-    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, 0x3000, 128, 1, 100, 512, 256, None) == -3
+    assert lib.lvx_cast_f32(0x1000, C.byref(t), 1, 8, 64, 64, 1, None) == -4
+    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, 1, None) == -3
+    assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, 2, None) == -1
+    assert lib.lvx_dx_vis(0x1000, 0x1100, 256, 0x2000, 0x3000, 250, 1, 0x4000, 512, 100, 512, 256, 1, None) == -2
+    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, 0x3000, 128, 1, 100, 512, 256, 1, None) == -3
     # the second operand pair is optional (single projection) but must be given or omitted as a pair
-    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, None, 256, 100, 512, 256, None) == -1
-    assert lib.lvx_dx_vis(0x1000, None, 256, 0x2000, 0x3000, 256, 1, 0x4000, 512, 100, 512, 256, None) == -1
-    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, None, 256, 1, 100, 512, 256, None) == -1
+    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, None, 256, 100, 512, 256, 1, None) == -1
+    assert lib.lvx_dx_vis(0x1000, None, 256, 0x2000, 0x3000, 256, 1, 0x4000, 512, 100, 512, 256, 1, None) == -1
+    assert lib.lvx_dw_kv(0x1000, 512, 0x1100, 0x1200, 256, 0x2000, None, 256, 1, 100, 512, 256, 1, None) == -1
     # the fused norm needs whole heads of 128 columns and its weight
     assert lib.lvx_kv_proj_norm(0x1000, 512, 0x2000, 0x3000, 192, 1, 0x4000, 0x5000, 192, 100, 512, 192,
-                                0x6000, 1e-5, None, None, None) == -4
+                                0x6000, 1e-5, None, None, 1, None) == -4
     assert lib.lvx_kv_proj_norm(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256,
-                                None, 1e-5, None, None, None) == -1
-    assert lib.lvx_k_norm_bwd(0x1000, 256, 0x2000, 256, None, 0x3000, 0x4000, 256, None, 100, 256, None) == -1
+                                None, 1e-5, None, None, 1, None) == -1
+    assert lib.lvx_k_norm_bwd(0x1000, 256, 0x2000, 256, None, 0x3000, 0x4000, 256, None, 100, 256, 1, None) == -1
+    # element types: 1 = bf16, 2 = fp16, anything else is refused
+    assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, 3, None) == -5
+    assert lib.lvx_cast_f32(0x1000, C.byref(t), 1, 8, 64, 128, 0, None) == -5
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _layer(impl):
+def _layer(impl, dtype=torch.bfloat16):
     from transformers.models.mllama import modeling_mllama as m
     from transformers.models.mllama.configuration_mllama import MllamaTextConfig
     cfg = MllamaTextConfig(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, num_hidden_layers=2,
@@ -22,11 +22,13 @@ def _layer(impl):
     with torch.no_grad():          # norm weights other than the all-ones initialisation
         layer.q_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
         layer.k_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
-    return layer.to(device=DEV, dtype=torch.bfloat16)
+    return layer.to(device=DEV, dtype=dtype)
 
 
-@pytest.mark.parametrize("variant", ["interface", "recompute", "recompute_intervals"])
-def test_mllama_cross_attention_layer_matches_eager(variant):
+@pytest.mark.parametrize("variant,dtype", [("interface", torch.bfloat16), ("recompute", torch.bfloat16),
+                                           ("recompute_intervals", torch.bfloat16),
+                                           ("interface", torch.float16), ("recompute", torch.float16)])
+def test_mllama_cross_attention_layer_matches_eager(variant, dtype):
     """interface: the attention-interface hook (K/V kept for backward);
     recompute: the patched forward (K/V + k_norm recomputed by the fused GEMM),
     with the dense mask or with the same mask as per-row key intervals."""
@@ -35,7 +37,7 @@ def test_mllama_cross_attention_layer_matches_eager(variant):
     from lv_xattn import _lib, hf_mllama
     _lib.load()
     name = hf_mllama.register()
-    ref, new = _layer("eager"), _layer(name)
+    ref, new = _layer("eager", dtype), _layer(name, dtype)
     new.load_state_dict(ref.state_dict())
     assert ref.head_dim == 128
     if variant != "interface":
@@ -43,13 +45,13 @@ def test_mllama_cross_attention_layer_matches_eager(variant):
 
     g = torch.Generator().manual_seed(11)
     B, Lq, Lkv = 2, 200, 1601
-    x = torch.randn(B, Lq, 1024, generator=g).bfloat16().to(DEV)
-    vis = torch.randn(B, Lkv, 1024, generator=g).bfloat16().to(DEV)
-    go = torch.randn(B, Lq, 1024, generator=g).bfloat16().to(DEV)
+    x = torch.randn(B, Lq, 1024, generator=g).to(dtype).to(DEV)
+    vis = torch.randn(B, Lkv, 1024, generator=g).to(dtype).to(DEV)
+    go = torch.randn(B, Lq, 1024, generator=g).to(dtype).to(DEV)
     # Llama-3.2 style additive mask: rows before the image see nothing (all entries
     # at the dtype minimum, as transformers builds it), sample 1 sees only the first tile
-    neg = torch.finfo(torch.bfloat16).min
-    mask = torch.zeros(B, 1, Lq, Lkv, dtype=torch.bfloat16)
+    neg = torch.finfo(dtype).min
+    mask = torch.zeros(B, 1, Lq, Lkv, dtype=dtype)
     mask[0, :, :17, :] = neg
     mask[1, :, :, 800:] = neg
     mask = mask.to(DEV)

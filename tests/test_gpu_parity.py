@@ -70,18 +70,19 @@ def test_kv_proj_dx_dw_small(lvx, w_in_major):
     check_grad(dwv, dwv_ref, "dW_v")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w_in_major", [True, False])
-def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major):
+def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major, dtype):
     from lv_xattn import ops
     g = torch.Generator().manual_seed(6)
     B, L, Dm, Hkv, D = 2, 301, 264, 4, 128          # ragged rows; 512 columns = two column tiles
-    x = (torch.randn(B, L, Dm, generator=g) * 0.5).bfloat16()
-    wk = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).bfloat16()
-    wv = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).bfloat16()
-    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).bfloat16()
+    x = (torch.randn(B, L, Dm, generator=g) * 0.5).to(dtype)
+    wk = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).to(dtype)
+    wv = (torch.randn(Dm, Hkv * D, generator=g) * 0.1).to(dtype)
+    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).to(dtype)
     eps = 1e-5
     k_raw_ref, v_ref = orc.kv_project(x, wk, wv, Hkv)
-    k_raw_ref = k_raw_ref.bfloat16()
+    k_raw_ref = k_raw_ref.to(dtype)
     k_ref = orc.k_rms_norm(k_raw_ref, wn, eps)
     wk_d, wv_d = (wk, wv) if w_in_major else (wk.t().contiguous(), wv.t().contiguous())
     k, v, k_raw, rstd = ops.kv_proj(_dev(x), _dev(wk_d), _dev(wv_d), Hkv, w_in_major, k_norm_weight=_dev(wn),
@@ -96,7 +97,7 @@ def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major):
     assert tuple(rstd.shape) == (B, L, Hkv)
     assert ((rstd.cpu() - r_ref).abs() <= 1e-2 * r_ref).all()
 
-    dk = torch.randn(B, L, Hkv, D, generator=g).bfloat16().transpose(1, 2)
+    dk = torch.randn(B, L, Hkv, D, generator=g).to(dtype).transpose(1, 2)
     dx_ref, dw_ref = orc.k_rms_norm_backward(dk, k_raw.float().cpu(), wn, eps)
     dk_raw, dw = ops.k_norm_bwd(_dev(dk.transpose(1, 2).contiguous()).transpose(1, 2), k_raw, rstd, _dev(wn))
     torch.cuda.synchronize()
@@ -104,21 +105,22 @@ def test_kv_proj_fused_k_norm_and_its_backward(lvx, w_in_major):
     check_grad(dw, dw_ref, "dw_norm")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w_in_major", [True, False])
-def test_q_projection_with_q_norm_autograd(lvx, w_in_major):
+def test_q_projection_with_q_norm_autograd(lvx, w_in_major, dtype):
     # the text side of `project`: Q = q_norm(X W_q), recomputed in backward
     g = torch.Generator().manual_seed(8)
     B, L, Dm, Hq, D = 2, 203, 328, 3, 128
-    x = (torch.randn(B, L, Dm, generator=g) * 0.5).bfloat16()
-    wq = (torch.randn(Dm, Hq * D, generator=g) * 0.1).bfloat16()
-    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).bfloat16()
-    dq = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    x = (torch.randn(B, L, Dm, generator=g) * 0.5).to(dtype)
+    wq = (torch.randn(Dm, Hq * D, generator=g) * 0.1).to(dtype)
+    wn = (1.0 + 0.3 * torch.randn(D, generator=g)).to(dtype)
+    dq = torch.randn(B, Hq, L, D, generator=g).to(dtype)
     q_raw_ref, _ = orc.kv_project(x, wq, wq, Hq)
-    q_raw_ref = q_raw_ref.bfloat16()
+    q_raw_ref = q_raw_ref.to(dtype)
     q_ref = orc.k_rms_norm(q_raw_ref, wn, 1e-5)
     dq_raw_ref, dwn_ref = orc.k_rms_norm_backward(dq, q_raw_ref, wn, 1e-5)
-    dx_ref = orc.dx_vis(dq_raw_ref.bfloat16(), torch.zeros_like(dq_raw_ref), wq, wq)
-    dw_ref, _ = orc.dw_kv(x, dq_raw_ref.bfloat16(), torch.zeros_like(dq_raw_ref))
+    dx_ref = orc.dx_vis(dq_raw_ref.to(dtype), torch.zeros_like(dq_raw_ref), wq, wq)
+    dw_ref, _ = orc.dw_kv(x, dq_raw_ref.to(dtype), torch.zeros_like(dq_raw_ref))
 
     proj = lvx.create_q_projection_class(w_in_major=w_in_major).apply
     xd = _dev(x).requires_grad_()
@@ -339,10 +341,13 @@ def test_recompute_layer_autograd(lvx, name):
     check_grad(wv.grad, dwv_ref, "dW_v")
 
 
-def test_recompute_layer_with_k_norm_autograd(lvx):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_recompute_layer_with_k_norm_autograd(lvx, dtype):
     w = orc.make_inputs(orc.workload("cfg2s"))
+    w.dtype = dtype
+    w.tensors = {n: (v.to(dtype) if v.is_floating_point() else v) for n, v in w.tensors.items()}
     t = w.tensors
-    wn = (1.0 + 0.3 * torch.randn(w.D, generator=torch.Generator().manual_seed(9))).bfloat16()
+    wn = (1.0 + 0.3 * torch.randn(w.D, generator=torch.Generator().manual_seed(9))).to(dtype)
     ref = orc.layer_reference(w, k_norm_weight=wn, k_norm_eps=1e-5)
     attention = lvx.create_attention_class("lv_xattn", rounds=w.rounds, weight_grads=True).apply
     q = _dev(t["q"]).requires_grad_()

@@ -42,18 +42,19 @@ def _piecewise_intervals(rng, B, Lq, Lkv, kv_len):
     return start, end
 
 
-def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided):
+def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided, dtype=torch.bfloat16,
+              sigma=1.0):
     D = 128
     scale = rng.choice([D ** -0.5, 0.05, 0.2])
     if strided:      # [B, S, H, D] memory viewed as [B, H, S, D]
-        q = torch.randn(B, Lq, Hq, D, generator=g).bfloat16().transpose(1, 2)
-        k = torch.randn(B, Lkv, Hkv, D, generator=g).bfloat16().transpose(1, 2)
-        v = torch.randn(B, Lkv, Hkv, D, generator=g).bfloat16().transpose(1, 2)
+        q = (sigma * torch.randn(B, Lq, Hq, D, generator=g)).to(dtype).transpose(1, 2)
+        k = (sigma * torch.randn(B, Lkv, Hkv, D, generator=g)).to(dtype).transpose(1, 2)
+        v = (sigma * torch.randn(B, Lkv, Hkv, D, generator=g)).to(dtype).transpose(1, 2)
     else:
-        q = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
-        k = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
-        v = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
-    do = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+        q = (sigma * torch.randn(B, Hq, Lq, D, generator=g)).to(dtype)
+        k = (sigma * torch.randn(B, Hkv, Lkv, D, generator=g)).to(dtype)
+        v = (sigma * torch.randn(B, Hkv, Lkv, D, generator=g)).to(dtype)
+    do = (sigma * torch.randn(B, Hq, Lq, D, generator=g)).to(dtype)
 
     kv_len = [Lkv] * B
     mask, allowed = None, None
@@ -68,11 +69,12 @@ def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, stri
             mask = lvx.Mask(kl, start, end)
         else:
             mask = lvx.Mask(kl)
-    what = f"B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv} P{rounds} batched={batched} mask={mask_kind} strided={strided}"
+    what = (f"B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv} P{rounds} batched={batched} mask={mask_kind} strided={strided} "
+            f"{dtype}")
     print(what, flush=True)
 
     o_ref, l_ref = orc.attention_dense(q, k, v, scale, allowed=allowed)
-    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.bfloat16(), l_ref, scale, allowed=allowed)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.to(dtype), l_ref, scale, allowed=allowed)
 
     qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
     _, _, _, o, L = lvx._attn_forward(qd, kd, vd, False, scale, None, rounds=rounds, mask=mask, batched=batched)
@@ -102,23 +104,40 @@ def test_random_shape_forward_backward(lvx, seed):
     _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided=seed % 3 == 0)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shape_forward_backward_fp16(lvx, seed):
+    # the reference's element type (lv_xattn/attn.py:226,250,268) with its harness' input scale
+    # (test.py:101-107: N(0, 0.5^2))
+    rng = random.Random(3000 + seed)
+    g = torch.Generator().manual_seed(4000 + seed)
+    B = rng.choice([1, 2])
+    Hq, Hkv = rng.choice([(4, 4), (8, 2), (8, 1), (6, 3)])
+    Lq = rng.randint(1, 600)
+    Lkv = rng.randint(2, 800)
+    rounds = rng.choice([1, 2, 4])
+    mask_kind = ["none", "kv_len", "intervals"][seed % 3]
+    _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, seed % 2 == 0, mask_kind, rng, g, strided=seed % 3 == 1,
+              dtype=torch.float16, sigma=0.5)
+
+
 @pytest.mark.parametrize("batched", [True, False])
 def test_more_than_four_runs_of_live_row_groups(lvx, batched):
     # 10 groups of 256 rows; group i sees only token block i % 2, so each of the two token
     # blocks is alive for five separate runs of row tiles
     B, Hq, Hkv, Lq, Lkv, D = 1, 2, 1, 2560, 256, 128
+    dtype, sigma = torch.bfloat16, 1.0
     g = torch.Generator().manual_seed(5)
-    q = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
-    k = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
-    v = torch.randn(B, Hkv, Lkv, D, generator=g).bfloat16()
-    do = torch.randn(B, Hq, Lq, D, generator=g).bfloat16()
+    q = (sigma * torch.randn(B, Hq, Lq, D, generator=g)).to(dtype)
+    k = (sigma * torch.randn(B, Hkv, Lkv, D, generator=g)).to(dtype)
+    v = (sigma * torch.randn(B, Hkv, Lkv, D, generator=g)).to(dtype)
+    do = (sigma * torch.randn(B, Hq, Lq, D, generator=g)).to(dtype)
     grp = torch.arange(Lq) // 256
     start = ((grp % 2) * 128 + 5).to(torch.int32)[None]
     end = ((grp % 2) * 128 + 120).to(torch.int32)[None]
     allowed = orc.interval_mask(start, end, Lkv)
     scale = D ** -0.5
     o_ref, l_ref = orc.attention_dense(q, k, v, scale, allowed=allowed)
-    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.bfloat16(), l_ref, scale, allowed=allowed)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.to(dtype), l_ref, scale, allowed=allowed)
     mask = lvx.Mask(None, start, end)
     qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
     rounds = 1 if batched else 2

@@ -58,10 +58,13 @@ def test_causal_and_malformed_bias_are_rejected_explicitly():
 
 
 def test_shape_and_dtype_checks_raise_before_any_device_call():
-    q = torch.zeros(1, 4, 8, 128, dtype=torch.float16)
-    k = torch.zeros(1, 2, 8, 128, dtype=torch.float16)
-    with pytest.raises(ops.LvxError, match="bf16"):
+    q = torch.zeros(1, 4, 8, 128, dtype=torch.float32)
+    k = torch.zeros(1, 2, 8, 128, dtype=torch.float32)
+    with pytest.raises(ops.LvxError, match="bf16 or fp16"):
         ops._shape(q, k, 0.1, None)
+    with pytest.raises(ops.LvxError, match="one type"):          # q and k of different 16-bit types
+        ops._shape(q.half(), k.bfloat16(), 0.1, None)
+    assert ops._shape(q.half(), k.half(), 0.1, None).dtype == 2 and ops._shape(q.bfloat16(), k.bfloat16(), 0.1, None).dtype == 1
     qb, kb = q.bfloat16(), torch.zeros(2, 2, 8, 128, dtype=torch.bfloat16)
     with pytest.raises(ops.LvxError, match="disagree"):
         ops._shape(qb, kb, 0.1, None)
