@@ -90,9 +90,12 @@ class Layer:
         self.out = dict(zip(("dq", "dk", "dv", "dx"), self.backward(k, v, o, L)), o=o, L=L)
 
 
-def time_gpu(fn, iters, warmup, torch):
-    """Median-free mean duration (ms) of fn over `iters` back-to-back calls,
-    measured with events on the stream the kernels are queued on."""
+def time_gpu(fn, iters, warmup, torch, stats=None):
+    """Mean duration (ms) of fn over `iters` back-to-back calls, measured with
+    two events on the stream the kernels are queued on.  `stats`, a dict, also
+    receives the median and the extremes of a second pass with an event between
+    every two calls (those events cost a few microseconds each, so the mean
+    comes from the first pass)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -102,6 +105,15 @@ def time_gpu(fn, iters, warmup, torch):
         fn()
     e1.record()
     torch.cuda.synchronize()
+    if stats is not None:
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
+        ev[0].record()
+        for i in range(iters):
+            fn()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ts = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(iters))
+        stats.update(median_ms=ts[iters // 2], min_ms=ts[0], max_ms=ts[-1])
     return e0.elapsed_time(e1) / iters
 
 
@@ -123,32 +135,41 @@ def kernel_breakdown(layer, n_pairs, torch):
     dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
     ops.bwd_preprocess(o, layer.do, delta)
     res = {}
-    it = 10
-    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=layer.mask), it, 3, torch)
-    res["fwd_all_rounds_one_launch"] = dict(ms=ms, tflops=f["fwd"] / ms / 1e9, frac_mfma=f["fwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+    it, wu = 30, 10      # launches timed / warm-up launches per operator
+    st = {}
+    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=layer.mask), it, wu, torch, st)
+    res["fwd_all_rounds_one_launch"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["fwd"] / ms / 1e9, frac_mfma=f["fwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
     lb = -(-Lq // w.rounds)
-    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask), it, 3, torch)
-    res["fwd_one_round"] = dict(ms=ms, tflops=f["fwd"] / w.rounds / ms / 1e9)
+    st = {}
+    ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask), it, wu, torch, st)
+    res["fwd_one_round"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["fwd"] / w.rounds / ms / 1e9)
     ws = torch.empty(ops.fwd_workspace_bytes(layer.q, k, lb, 4), dtype=torch.uint8, device=dev)
+    st = {}
     ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, 0, lb, mask=layer.mask, kv_splits=4,
-                                  workspace=ws), it, 3, torch)
-    res["fwd_one_round_4_key_splits"] = dict(ms=ms, tflops=f["fwd"] / w.rounds / ms / 1e9)
+                                  workspace=ws), it, wu, torch, st)
+    res["fwd_one_round_4_key_splits"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["fwd"] / w.rounds / ms / 1e9)
+    st = {}
     ms = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask,
-                                  workspace=bws), it, 3, torch)
-    res["bwd_all_rounds_one_launch"] = dict(ms=ms, tflops=f["bwd"] / ms / 1e9, frac_mfma=f["bwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+                                  workspace=bws), it, wu, torch, st)
+    res["bwd_all_rounds_one_launch"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["bwd"] / ms / 1e9, frac_mfma=f["bwd"] / ms / 1e9 / PEAK_BF16_TFLOPS)
     merge_bytes = (3 * D * 2 + 3 * 4) * B * Hq * Lq
-    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L), it, 3, torch)
-    res["merge_all_rounds_one_launch"] = dict(ms=ms, gbs=merge_bytes / ms / 1e6, frac_hbm=merge_bytes / ms / 1e6 / PEAK_HBM_GBS)
-    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L, 0, lb), it, 3, torch)
-    res["merge_one_round"] = dict(ms=ms, gbs=merge_bytes / w.rounds / ms / 1e6)
+    st = {}
+    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L), it, wu, torch, st)
+    res["merge_all_rounds_one_launch"] = dict(ms=ms, median_ms=st["median_ms"], gbs=merge_bytes / ms / 1e6, frac_hbm=merge_bytes / ms / 1e6 / PEAK_HBM_GBS)
+    st = {}
+    ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L, 0, lb), it, wu, torch, st)
+    res["merge_one_round"] = dict(ms=ms, median_ms=st["median_ms"], gbs=merge_bytes / w.rounds / ms / 1e6)
     pre_bytes = (2 * D * 2 + 4) * B * Hq * Lq
-    ms = time_gpu(lambda: ops.bwd_preprocess(o, layer.do, delta), it, 3, torch)
-    res["preprocess"] = dict(ms=ms, gbs=pre_bytes / ms / 1e6, frac_hbm=pre_bytes / ms / 1e6 / PEAK_HBM_GBS)
+    st = {}
+    ms = time_gpu(lambda: ops.bwd_preprocess(o, layer.do, delta), it, wu, torch, st)
+    res["preprocess"] = dict(ms=ms, median_ms=st["median_ms"], gbs=pre_bytes / ms / 1e6, frac_hbm=pre_bytes / ms / 1e6 / PEAK_HBM_GBS)
     if layer.has_proj:
-        ms = time_gpu(lambda: layer.project(), it, 3, torch)
-        res["kv_proj"] = dict(ms=ms, tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
-        ms = time_gpu(lambda: ops.dx_vis(dk, dv, layer.wk, layer.wv), it, 3, torch)
-        res["dx_vis"] = dict(ms=ms, tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+        st = {}
+        ms = time_gpu(lambda: layer.project(), it, wu, torch, st)
+        res["kv_proj"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
+        st = {}
+        ms = time_gpu(lambda: ops.dx_vis(dk, dv, layer.wk, layer.wv), it, wu, torch, st)
+        res["dx_vis"] = dict(ms=ms, median_ms=st["median_ms"], tflops=f["proj"] / ms / 1e9, frac_mfma=f["proj"] / ms / 1e9 / PEAK_BF16_TFLOPS)
     for d in res.values():
         for key in d:
             d[key] = round(d[key], 5)
