@@ -104,6 +104,23 @@ def test_random_shape_forward_backward(lvx, seed):
     _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided=seed % 3 == 0)
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_random_shape_few_rows_many_keys(lvx, seed):
+    # few rows against a long shard: the forward cuts the key range into splits folded by the
+    # merge kernel, the backward splits the dQ contraction over the tokens
+    from lv_xattn.attn import auto_kv_splits
+    rng = random.Random(5000 + seed)
+    g = torch.Generator().manual_seed(6000 + seed)
+    B = rng.choice([1, 2])
+    Hq, Hkv = rng.choice([(4, 2), (8, 2), (4, 4)])
+    Lq = rng.randint(1, 120)
+    Lkv = rng.randint(1100, 2600)
+    assert auto_kv_splits(B, Hq, Hkv, Lq, Lkv) > 1
+    mask_kind = ["none", "intervals", "kv_len", "intervals"][seed]
+    _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rng.choice([1, 2]), seed % 2 == 0, mask_kind, rng, g, strided=seed == 3,
+              dtype=[torch.bfloat16, torch.float16][seed % 2], sigma=[1.0, 0.5][seed % 2])
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_shape_forward_backward_fp16(lvx, seed):
     # the reference's element type (lv_xattn/attn.py:226,250,268) with its harness' input scale
