@@ -81,8 +81,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const int sp = wid % p.q_splits;
     const int kblk = (wid / p.q_splits) % p.n_kv_blocks;
     const int bh = wid / (p.q_splits * p.n_kv_blocks);
-    const int hk = bh % p.Hkv;
-    const int b = bh / p.Hkv;
+    const int b = bh % p.B;            // samples interleaved: ragged samples then share the tail of the launch
+    const int hk = bh / p.B;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
