@@ -97,21 +97,6 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const bool kv_valid = my_kv < kv_len;
     const bool tail_block = kvb + BN > kv_len;
 
-    // ---- resident B operand: this wave's K rows (P-wave) or V rows (D-wave)
-    bf16x8 breg[8];
-    {
-        const uint16_t* base = d_role ? p.v + b * p.vs.b + hk * p.vs.h + (int64_t)my_kv * p.vs.s
-                                      : p.k + b * p.ks.b + hk * p.ks.h + (int64_t)my_kv * p.ks.s;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) breg[kk] = as_bf16x8(ldg16(base + kk * 16 + g * 8, kv_valid));
-    }
-    // ---- resident accumulator: dV^T (P-wave) or dK^T (D-wave), [128 d][32 tokens]
-    f32x16 acc[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
-
     // steps of this work-group: a contiguous range of the (head, row tile) list
     const int n_qtiles = (p.row_end - p.row_begin + BM - 1) / BM;
     // with an interval mask only the listed runs of tiles are visited (kept in scalar
@@ -131,6 +116,24 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     auto sel4 = [](int r, const int (&a)[4]) { return r == 0 ? a[0] : r == 1 ? a[1] : r == 2 ? a[2] : a[3]; };
     const int it_lo = sp * split_steps;
     const int n_iter = (kvb < kv_len) ? max(0, min(split_steps, p.G * n_live - it_lo)) : 0;
+    // nothing to visit and nothing to overwrite: done (bf16 outputs, mode 0, still get their zeros)
+    if (n_iter == 0 && p.dkv_mode != 0) return;
+
+    // ---- resident B operand: this wave's K rows (P-wave) or V rows (D-wave)
+    bf16x8 breg[8];
+    {
+        const uint16_t* base = d_role ? p.v + b * p.vs.b + hk * p.vs.h + (int64_t)my_kv * p.vs.s
+                                      : p.k + b * p.ks.b + hk * p.ks.h + (int64_t)my_kv * p.ks.s;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) breg[kk] = as_bf16x8(ldg16(base + kk * 16 + g * 8, kv_valid));
+    }
+    // ---- resident accumulator: dV^T (P-wave) or dK^T (D-wave), [128 d][32 tokens]
+    f32x16 acc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+
     const float c = p.scale_log2e;
 
     // global -> LDS is the P-waves' job (their step is the shorter one): P-wave w moves
