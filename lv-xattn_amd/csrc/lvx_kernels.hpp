@@ -120,10 +120,6 @@ struct MetaParams {
     int meta_blocks;           // filled by the launcher: blocks [0, meta_blocks) write records
 };
 
-struct FillParams {
-    uint32_t* dst;             // 16-byte aligned
-    int64_t n16;               // number of 16-byte chunks to zero
-};
 
 struct CastParams {
     const float* src;
@@ -192,7 +188,6 @@ hipError_t launch_preprocess(const PreParams& p, hipStream_t st);
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st);
 hipError_t launch_cast(const CastParams& p, hipStream_t st);
 hipError_t launch_bwd_meta(const MetaParams& p, hipStream_t st);
-hipError_t launch_zero(const FillParams& p, hipStream_t st);
 
 // Backward of the 128-wide RMS norm: rows of dy, x [M][heads][128] (row strides ldy, ldx), r [M][heads].
 struct NormBwdParams {

@@ -123,7 +123,9 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
 // window (so that P = exp2(x - inf) = 0 there), and delta * scale (0 past the
 // window), grouped per 32-row tile so that one 256-byte load fetches a tile's lot.
 __global__ __launch_bounds__(256) void bwd_meta_kernel(const MetaParams p) {
-    if ((int)blockIdx.x >= p.meta_blocks) {   // the other blocks of the launch zero the scratches
+    // the other blocks of the launch zero the scratches (stores rather than hipMemsetAsync, so
+    // that callers may capture the stream)
+    if ((int)blockIdx.x >= p.meta_blocks) {
         const u32x4 z = {0u, 0u, 0u, 0u};
         const int64_t first = (int64_t)(blockIdx.x - p.meta_blocks) * 256 + threadIdx.x;
         const int64_t stride = (int64_t)(gridDim.x - p.meta_blocks) * 256;
@@ -291,13 +293,6 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const NormBwdParams p) {
     }
 }
 
-// zero fill (a kernel rather than hipMemsetAsync, so that callers may capture the stream)
-__global__ __launch_bounds__(256) void zero_kernel(const FillParams p) {
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < p.n16; i += (int64_t)gridDim.x * 256)
-        reinterpret_cast<u32x4*>(p.dst)[i] = z;
-}
-
 inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 
 }  // namespace
@@ -335,13 +330,6 @@ hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), 0, st, p);
-    return hipGetLastError();
-}
-
-hipError_t launch_zero(const FillParams& p, hipStream_t st) {
-    if (p.n16 <= 0) return hipSuccess;
-    const int grid = (int)((p.n16 + 255) / 256 < 4096 ? (p.n16 + 255) / 256 : 4096);
-    hipLaunchKernelGGL(zero_kernel, dim3(grid), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 
