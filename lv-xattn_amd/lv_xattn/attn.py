@@ -110,12 +110,11 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     if mask is not None:
         mask = mask.to(dev)
 
-    if acc_in is None:
-        o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
-        L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
-    else:
-        o = acc_in[0].to(dtype=q_.dtype).clone(memory_format=torch.contiguous_format)
-        L = acc_in[1].to(torch.float32).reshape(B * Hq, Lq).clone()
+    o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
+    L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
+    if acc_in is not None:
+        acc_o = _usable(acc_in[0].to(dtype=q_.dtype))
+        acc_l = acc_in[1].to(torch.float32).reshape(B * Hq, Lq).contiguous()
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
     max_rows = max(r1 - r0 for r0, r1 in windows)
@@ -126,16 +125,13 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
         nbytes = ops.fwd_workspace_bytes(q_, k_, max_rows, kv_splits)
         ws = workspace("fwd_split", (nbytes,), torch.uint8, dev)
 
-    if acc_in is None:
-        # merging into the identity returns the partial itself: write in place
-        for r0, r1 in windows:
-            ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
-    else:
-        o_part = workspace("fwd_o_part", (B, Hq, Lq, D), q_.dtype, dev)
-        l_part = workspace("fwd_l_part", (B * Hq, Lq), torch.float32, dev)
-        for r0, r1 in windows:
-            ops.fwd(q_, k_, v_, o_part, l_part, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
-            ops.merge(o, L, o_part, l_part, r0, r1 - r0)
+    # the partial goes straight into (o, L); an incoming accumulator is then folded into it
+    # (the merge is symmetric, so which side is "the accumulator" does not matter, and neither
+    # a copy of acc_in nor a buffer for the partial is needed)
+    for r0, r1 in windows:
+        ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
+        if acc_in is not None:
+            ops.merge(o, L, acc_o, acc_l, r0, r1 - r0)
     return q, k, v, o, L
 
 
