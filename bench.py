@@ -209,10 +209,15 @@ def run_only(layer, which, n, torch):
     else:
         fn = lambda: ops.dx_vis(k, v, layer.wk, layer.wv)
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
     for _ in range(n):
         fn()
+    e1.record()
     torch.cuda.synchronize()
-    print(json.dumps({"only": which, "launches": n, "workload": w.name}))
+    # the same launches as the profiler sees them, timed with events on their stream
+    print(json.dumps({"only": which, "launches": n, "workload": w.name,
+                      "avg_launch_ms": round(e0.elapsed_time(e1) / n, 5)}))
 
 
 def cpu_baseline(w, budget_rounds=8):
@@ -260,8 +265,8 @@ def cpu_baseline(w, budget_rounds=8):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)   # ~45 ms: the clocks settle after ~40 ms of load
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--mode", default="batched", choices=["batched", "rounds"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
