@@ -95,3 +95,12 @@ def test_llama_cross_attention_mask_to_intervals():
     # a gap (image 0 with 2 of 4 tiles, then image 1) has no interval form
     cam[0, 5, 0, :2] = 1
     assert mask_from_cross_attention_mask(cam, 5) is None
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "single-GPU" in (r.stderr + r.stdout)
