@@ -41,6 +41,23 @@ def _usable(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+HEAD_DIM = 128          # the head dimension the kernels are built for
+
+
+def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
+    """Smaller head dimensions run zero-padded to 128: the padded columns add
+    nothing to q k^T, and the padded columns of O, dQ, dK and dV come out zero
+    and are cut off again.  Exact, at the cost of the padded arithmetic."""
+    D = t.shape[-1]
+    if D == HEAD_DIM:
+        return t
+    if D > HEAD_DIM:
+        raise ValueError(f"head_dim {D} exceeds {HEAD_DIM}")
+    out = t.new_zeros(*t.shape[:-1], HEAD_DIM)
+    out[..., :D] = t
+    return out
+
+
 def _reject_unsupported(causal):
     if causal:
         # the reference applies the triangle to rank-local indices only
@@ -102,7 +119,8 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     work-groups, see auto_kv_splits), `batched` (one launch over all P blocks
     instead of one per round)."""
     _reject_unsupported(causal)
-    q_, k_, v_ = _usable(q), _usable(k), _usable(v)
+    D_in = q.shape[-1]
+    q_, k_, v_ = (_usable(_pad_head_dim(t)) for t in (q, k, v))
     B, Hq, Lq, D = q_.shape
     P = rounds if rounds is not None else get_sequence_parallel_size()
     dev = q_.device
@@ -113,7 +131,7 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
     L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
     if acc_in is not None:
-        acc_o = _usable(acc_in[0].to(dtype=q_.dtype))
+        acc_o = _usable(_pad_head_dim(acc_in[0].to(dtype=q_.dtype)))
         acc_l = acc_in[1].to(torch.float32).reshape(B * Hq, Lq).contiguous()
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
@@ -132,6 +150,8 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
         ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
         if acc_in is not None:
             ops.merge(o, L, acc_o, acc_l, r0, r1 - r0)
+    if D_in != D:
+        o = o[..., :D_in].contiguous()
     return q, k, v, o, L
 
 
@@ -147,7 +167,8 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     complete after that round (fp32 sum over all local tokens, rounded once).
     `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored."""
     _reject_unsupported(causal)
-    q_, k_, v_, o_, do_ = (_usable(t) for t in (q, k, v, o, do))
+    D_in = q.shape[-1]
+    q_, k_, v_, o_, do_ = (_usable(_pad_head_dim(t)) for t in (q, k, v, o, do))
     B, Hq, Lq, D = q_.shape
     Hkv, Lkv = k_.shape[1], k_.shape[2]
     P = rounds if rounds is not None else get_sequence_parallel_size()
@@ -182,4 +203,8 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
         # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
         ops.cast_f32(dk_acc.transpose(1, 2), dk.transpose(1, 2))
         ops.cast_f32(dv_acc.transpose(1, 2), dv.transpose(1, 2))
+    if D_in != D:
+        dq = dq[..., :D_in].contiguous()
+        dk = dk.transpose(1, 2)[..., :D_in].contiguous().transpose(1, 2)
+        dv = dv.transpose(1, 2)[..., :D_in].contiguous().transpose(1, 2)
     return dq, dk, dv

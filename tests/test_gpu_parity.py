@@ -288,6 +288,52 @@ def test_backward_cfg1s(lvx, batched):
     check_grad(dv, ref["dv"], "dV")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batched", [False, True])
+def test_cfg0_shape_head_dim_64_runs_zero_padded(lvx, batched, dtype):
+    """The CPU-only fp32 workload (head_dim 64, 4 rounds of 32 rows, 4096 keys) at its own
+    shape, rounded to a 16-bit type: smaller head dimensions run zero-padded to 128 in the host
+    loops, outputs and gradients come back at 64 columns."""
+    w = orc.make_inputs(orc.workload("cfg0"))
+    assert w.D == 64 and abs(w.scale - 0.125) < 1e-12
+    w.dtype = dtype
+    w.tensors = {n: x.to(dtype) for n, x in w.tensors.items()}
+    t = w.tensors
+    ref = orc.layer_reference(w)
+    q, k, v, do = (_dev(t[n]) for n in ("q", "k", "v", "do"))
+    _, _, _, o, L = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, batched=batched)
+    dq, dk, dv = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash",
+                                    rounds=w.rounds, batched=batched)
+    torch.cuda.synchronize()
+    assert o.shape == q.shape and o.is_contiguous() and o.dtype == dtype
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    check_o(o, ref["o"])
+    check_lse(L, ref["lse"].reshape(w.B * w.Hq, w.Lq))
+    check_grad(dq, ref["dq"], "dQ")
+    check_grad(dk, ref["dk"], "dK")
+    check_grad(dv, ref["dv"], "dV")
+
+
+def test_head_dim_80_with_incoming_accumulator(lvx):
+    """Any head dimension up to 128 pads; the incoming accumulator pads with it."""
+    g = torch.Generator().manual_seed(31)
+    B, Hq, Hkv, D, Lq, Lkv = 2, 4, 2, 80, 96, 700
+    q, k, v = (torch.randn(B, h, l, D, generator=g).bfloat16() for h, l in ((Hq, Lq), (Hkv, Lkv), (Hkv, Lkv)))
+    k2, v2 = (torch.randn(B, Hkv, 300, D, generator=g).bfloat16() for _ in range(2))
+    scale = D ** -0.5
+    o_in, l_in = orc.attention_dense(q, k2, v2, scale)
+    o_ref, l_ref = orc.attention_dense(q, torch.cat([k, k2], 2), torch.cat([v, v2], 2), scale)
+    _, _, _, o, L = lvx._attn_forward(_dev(q), _dev(k), _dev(v), False, scale, None, rounds=3,
+                                      acc_in=(_dev(o_in.bfloat16()), _dev(l_in.reshape(B * Hq, Lq))))
+    torch.cuda.synchronize()
+    assert o.shape == (B, Hq, Lq, D)
+    check_o(o, o_ref)
+    check_lse(L, l_ref.reshape(B * Hq, Lq))
+    with pytest.raises(ValueError, match="exceeds 128"):
+        lvx._attn_forward(_dev(torch.zeros(1, 2, 32, 160).bfloat16()), _dev(torch.zeros(1, 2, 64, 160).bfloat16()),
+                          _dev(torch.zeros(1, 2, 64, 160).bfloat16()), False, 0.1, None, rounds=1)
+
+
 @pytest.mark.parametrize("batched", [False, True])
 def test_backward_masked_ragged_cfg4s(lvx, batched):
     w = orc.make_inputs(orc.workload("cfg4s"))
