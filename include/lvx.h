@@ -127,7 +127,7 @@ int lvx_bwd_preprocess(const lvx_attn_shape* shape, const lvx_tensor* o, const l
  *            dkv_accumulate == 1: fp32 tensors of the same indexing, added to;
  *   workspace : lvx_bwd_workspace_bytes(shape, row_count) bytes, 16-byte
  *            aligned; holds scale*dS (16-bit) between the kernels of the call, the row
- *            metadata and, for small windows, fp32 partial sums of dK/dV and dQ.
+ *            metadata and, for small windows, fp32 partial sums of dK/dV and partial tiles of dQ.
  */
 int lvx_bwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
             const lvx_tensor* v, const lvx_tensor* dout, const float* lse, const float* delta,

@@ -239,9 +239,10 @@ static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
 }
 
 // The dQ GEMM of a small row window (a one-round launch) has only B*Hq C tiles; its
-// contraction over the tokens is then split over several work-groups that add fp32
-// partial tiles into a scratch, rounded to bf16 afterwards.  Returns the number of
-// splits (1: none) and the tokens per split.
+// contraction over the tokens is then split over several work-groups that store fp32
+// partial tiles, each split into its own slice of a scratch; the slices are summed and
+// rounded to bf16 afterwards (fp32 atomics into one slice were measured slower).  Returns
+// the number of splits (1: none) and the tokens per split.
 static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_len) {
     const int tile_rows = s->kv_start ? 256 : 512;      // as launch_gemm picks them
     const int tiles = row_count > 256 ? (row_count + tile_rows - 1) / tile_rows : 1;
@@ -255,8 +256,8 @@ static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_le
 }
 
 // Regions of the backward workspace, in order: dS^T tiles; fp32 dK/dV scratch (split-steps mode
-// with bf16 outputs); row metadata records (2 floats per row and head); fp32 dQ partial sums
-// (split dQ contraction only); with an interval mask the live-tile tables (group hulls, runs
+// with bf16 outputs); row metadata records (2 floats per row and head); fp32 dQ partial tiles,
+// one slice per split (split dQ contraction only); with an interval mask the live-tile tables (group hulls, runs
 // of live tiles per token block).  Every region is a multiple of 16 bytes.
 struct BwdWorkspace {
     size_t ds, dkv, meta, dq32, hull, runs, total;
@@ -277,7 +278,8 @@ static BwdWorkspace bwd_workspace(const lvx_attn_shape* s, int32_t row_count) {
     w.meta = off; off += (size_t)s->B * s->Hq * rows * 2 * sizeof(float);
     int sl;
     w.dq32 = off;
-    if (dq_k_splits(s, row_count, &sl) > 1) off += (size_t)s->B * s->Hq * rows * s->D * sizeof(float);
+    const int ks = dq_k_splits(s, row_count, &sl);
+    if (ks > 1) off += (size_t)ks * s->B * s->Hq * rows * s->D * sizeof(float);
     if (s->kv_start) {
         const size_t nkb = tokens / 128;
         w.hull = off; off += up16((size_t)s->B * w.n_groups * 2 * sizeof(int32_t));
@@ -354,8 +356,6 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         MetaParams mp{lse, delta, meta, s->B, s->Hq, s->Lq, row_begin, row_begin + row_count, (int)(rows / 32), s->scale};
         mp.zero_dst[0] = reinterpret_cast<uint32_t*>(scratch);
         mp.zero_n16[0] = scratch ? (int64_t)(dkv_scratch_bytes(s) / 16) : 0;
-        mp.zero_dst[1] = reinterpret_cast<uint32_t*>(dq32);
-        mp.zero_n16[1] = dq32 ? (int64_t)s->B * s->Hq * rows * s->D * (int64_t)sizeof(float) / 16 : 0;
         hipError_t em = launch_bwd_meta(mp, st);
         if (em != hipSuccess) return static_cast<int>(em);
         p.meta = meta;
@@ -417,9 +417,11 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.k_range = hull;            // [B][M tiles][2]: the group hulls are per M tile of this GEMM
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
     if (ks <= 1) return static_cast<int>(launch_gemm(g, true, true, st));
-    // split contraction: accumulate in the (already zeroed) fp32 scratch, round into dq
+    // split contraction: every split stores its partial tiles in its own fp32 slice; the
+    // cast sums the slices and rounds into dq
     g.k_splits = ks; g.k_split_len = split_len;
-    g.c32 = dq32; g.c32_batch = (int64_t)row_count * s->D; g.c32_ld = row_count;   // [B * Hq][D][row_count]
+    g.c32 = dq32; g.c32_batch = (int64_t)row_count * s->D; g.c32_ld = row_count;   // [split][B * Hq][D][row_count]
+    g.c32_split = (int64_t)s->B * s->Hq * g.c32_batch;
     e = launch_gemm(g, true, true, st);
     if (e != hipSuccess) return static_cast<int>(e);
     CastParams cq{};
@@ -429,6 +431,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     cq.ds = st3(dq);
     cq.B = s->B; cq.H = s->Hq; cq.L = row_count;
     cq.transposed = 1;
+    cq.nsum = ks; cq.sum_stride = g.c32_split;
     return static_cast<int>(launch_cast(cq, st));
 }
 

@@ -251,9 +251,8 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     if (set == 0) phase_barrier();
 
     // C^T tile: accumulator rows = n, cols = m
-    if (nks > 1) {   // partial tile of a split contraction: fp32 atomic adds
-        if (steps == 0) return;
-        float* const C32 = p.c32 + (int64_t)z * p.c32_batch;
+    if (nks > 1) {   // partial tile of a split contraction: fp32, into this split's slice
+        float* const C32 = p.c32 + ksp * p.c32_split + (int64_t)z * p.c32_batch;
 #pragma unroll
         for (int mt = 0; mt < WM; ++mt) {
             const int m = m0 + 32 * (WM * wm + mt) + l32;
@@ -265,7 +264,7 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
                     const int n = n0 + 32 * (WN * wn + nt) + 8 * vg + 4 * g;
                     if (n < p.N) {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) unsafeAtomicAdd(C32 + (int64_t)(n + r) * p.c32_ld + m, acc[nt][mt][4 * vg + r]);
+                        for (int r = 0; r < 4; ++r) C32[(int64_t)(n + r) * p.c32_ld + m] = acc[nt][mt][4 * vg + r];
                     }
                 }
         }

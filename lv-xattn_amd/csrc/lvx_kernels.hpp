@@ -127,6 +127,8 @@ struct CastParams {
     Strides3 ds;
     int B, H, L;
     int transposed;   // 0: src is [B*H][L][D]; 1: src is [B*H][D][L]
+    int nsum;         // transposed only: the result is the sum of nsum such sources (0 or 1: one),
+    int64_t sum_stride;   // sum_stride floats apart
     int f16;          // destination type: 0 bf16, 1 fp16
 };
 
@@ -169,13 +171,15 @@ struct GemmParams {
     const int32_t* k_range;
     int f16;                   // element type of A, B, C (and the norm weight): 0 bf16, 1 fp16
     // Split contraction (single-segment problems): k_splits work-groups per C tile, each
-    // contracting k_split_len values of k (a multiple of 128) and adding its partial tile
-    // with fp32 atomics to the TRANSPOSED scratch c32[z * c32_batch + n * c32_ld + m] (zeroed
-    // by the caller; the accumulator holds C^T, so a wave's lanes then add to consecutive
-    // addresses) instead of storing bf16 to C.  k_splits <= 1: off.
+    // contracting k_split_len values of k (a multiple of 128) and storing its partial tile
+    // in fp32 to its own slice of the TRANSPOSED scratch
+    // c32[split * c32_split + z * c32_batch + n * c32_ld + m] (the accumulator holds C^T, so
+    // a wave's lanes then write consecutive addresses; every split writes its whole tile,
+    // zeros if its range is empty) instead of storing bf16 to C; the caller sums the slices.
+    // k_splits <= 1: off.
     int k_splits, k_split_len;
     float* c32;
-    int64_t c32_batch;
+    int64_t c32_split, c32_batch;
     int c32_ld;
     // a_tiled_m > 0: A (stored [K][M]) is cut into contiguous [128 k][32 m] tiles,
     // a_tiled_m of them per block of 128 k; lda is ignored

@@ -214,8 +214,8 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
 }
 
-// Same from a transposed source [B*H][D][L]: adjacent threads take adjacent rows, so the
-// eight strided reads of a thread are coalesced across the wave.
+// Same from a transposed source [B*H][D][L], or the sum of several: adjacent threads take
+// adjacent rows, so the eight strided reads of a thread are coalesced across the wave.
 template <bool F16>
 __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
     using E = Elt<F16>;
@@ -229,6 +229,11 @@ __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
     float a[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) a[j] = s[(int64_t)j * p.L];
+    for (int k = 1; k < p.nsum; ++k) {
+        s += p.sum_stride;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] += s[(int64_t)j * p.L];
+    }
     u32x4 u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) u[j] = E::pack(a[2 * j], a[2 * j + 1]);

@@ -98,8 +98,9 @@ def test_other_entry_points_reject_bad_arguments(lib):
                        C.byref(t), C.byref(t), 2, 0, 64, 0x4000, 1 << 30, None) == -3
     need = lib.lvx_bwd_workspace_bytes(C.byref(s), 64)
     # dS^T tiles + fp32 dK/dV scratch + row metadata records (2 floats per row and head)
-    # + fp32 dQ partial sums (a window this small splits the dQ contraction over the tokens)
-    assert need == 8 * 256 * 64 * 2 + 2 * 256 * 2 * 128 * 4 + 8 * 64 * 2 * 4 + 8 * 64 * 128 * 4
+    # + fp32 dQ partial tiles (a window this small splits the dQ contraction over the tokens:
+    # 2 token blocks, one slice each)
+    assert need == 8 * 256 * 64 * 2 + 2 * 256 * 2 * 128 * 4 + 8 * 64 * 2 * 4 + 2 * 8 * 64 * 128 * 4
     # an interval mask adds the live-tile tables: one hull (2 ints, padded to 16 bytes) for the
     # single 256-row group and 8 ints per token block
     sm = _shape(kv_start=0x3000, kv_end=0x3100)
