@@ -216,14 +216,13 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
 // (which then add their dK/dV with atomics) evens that out; S is chosen to
 // minimise ceil(blocks * S / CUs) / S with ranges of at least 32 steps.
 static int choose_q_splits(int blocks, int steps) {
-    static int n_cu = 0;
-    if (n_cu == 0) {
-        int dev = 0;
+    static const int n_cu = [] {      // initialised once, by whichever thread comes first
+        int dev = 0, n = 0;
         hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n_cu = prop.multiProcessorCount;
-        if (n_cu <= 0) n_cu = 256;
-    }
+            n = prop.multiProcessorCount;
+        return n > 0 ? n : 256;
+    }();
     int best = 1;
     double best_cost = (double)((blocks + n_cu - 1) / n_cu);
     for (int S = 2; S <= 8; ++S) {

@@ -95,6 +95,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const int kvb = kblk * BN;
     const int my_kv = kvb + 32 * slice + l32;
     const bool kv_valid = my_kv < kv_len;
+    const int slice_lo = kvb + 32 * slice;              // this wave's 32 tokens
+    const bool slice_valid = slice_lo + 32 <= kv_len;   // all of them inside the sample
     const bool tail_block = kvb + BN > kv_len;
 
     // steps of this work-group: a contiguous range of the (head, row tile) list
@@ -259,6 +261,14 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         const char* dot = reinterpret_cast<const char*>(tile_prev) + TILE_ELEMS * 2;
         bf16x8 qa[8];
         u32x2 da[4][2][2];
+        // MASKED: lane l looks at the key interval of row l of the previous tile (requested
+        // first, so the answer is there long before it is needed)
+        int iv_s = 0, iv_e = 0;
+        if (MASKED && pv_live) {
+            const int32_t* iv = reinterpret_cast<const int32_t*>(meta + 16);
+            iv_s = iv[l32];
+            iv_e = iv[32 + l32];
+        }
         if (s_live) {
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk)
@@ -293,14 +303,19 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 }
             }
             if (MASKED) {
+                // most (tile, token slice) pairs a mask leaves alive are alive as a whole; only a
+                // slice that some row of the tile cuts is masked element by element
+                const bool cut = iv_s > slice_lo || iv_e < slice_lo + 32;
+                if (!slice_valid || __builtin_amdgcn_ballot_w64(cut) != 0) {
 #pragma unroll
-                for (int vg = 0; vg < 4; ++vg) {
-                    const u32x4 sp = meta[16 + 2 * vg + g];
-                    const u32x4 ep = meta[24 + 2 * vg + g];
+                    for (int vg = 0; vg < 4; ++vg) {
+                        const u32x4 sp = meta[16 + 2 * vg + g];
+                        const u32x4 ep = meta[24 + 2 * vg + g];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
-                        s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
+                        for (int r = 0; r < 4; ++r) {
+                            const bool vis = kv_valid && my_kv >= (int)sp[r] && my_kv < (int)ep[r];
+                            s[4 * vg + r] = vis ? s[4 * vg + r] : 0.f;
+                        }
                     }
                 }
             } else if (TAIL) {
