@@ -47,8 +47,10 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     and the subtraction stays accurate.  A row that is masked everywhere then
     attends by its scores over the masked keys (as it does in the reference,
     whose fp16 fill value is -65504; transformers' eager path attends uniformly
-    there) - the Mllama decoder layer zeroes such rows right after the
-    attention (full_text_row_masked_out_mask), so the difference never shows."""
+    there).  The masks transformers builds hold no such row: its
+    _prepare_cross_attention_mask multiplies the mask by
+    full_text_row_masked_out_mask, which turns a row that sees no tile into a
+    row that sees every key."""
     return mask.float().clamp_min(-30000.0)
 
 
@@ -58,10 +60,13 @@ def lv_xattn_attention_forward(module, query, key, value, attention_mask: Option
     eager_attention_forward): returns (attn_output [B, Lq, Hq, D], None)."""
     global _attention
     if kwargs.get("is_causal", False) or getattr(module, "is_causal", False) is True or not hasattr(module, "k_norm"):
-        # a (causal) self-attention layer: another operator, transformers' own
-        from transformers.models.mllama.modeling_mllama import eager_attention_forward
-        return eager_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
-                                       scaling=scaling, **kwargs)
+        # a (causal) self-attention layer: another operator, transformers' own.  Its SDPA
+        # form, because the masks this implementation name is registered with (see register)
+        # are SDPA masks: None stands for "plain causal", which eager attention would read
+        # as "no mask at all".
+        from transformers.integrations.sdpa_attention import sdpa_attention_forward
+        return sdpa_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
+                                      scaling=scaling, **kwargs)
     _require_supported(query, key, dropout)
     if _attention is None:
         _attention = create_attention_class_save_qkv("lv_xattn", rounds=1, batched=True).apply
@@ -146,11 +151,16 @@ def register() -> str:
     its name.  Raises ImportError if transformers has no attention interface."""
     from transformers import AttentionInterface
     AttentionInterface.register(NAME, lv_xattn_attention_forward)
+    # The registry is model-wide: the self-attention layers get their masks by this name too.
+    # Without an entry transformers builds no mask at all for a custom implementation (padding
+    # included), so the name is given the SDPA mask builder.
+    from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+    AttentionMaskInterface.register(NAME, sdpa_mask)
     return NAME
 
 
 def mask_from_cross_attention_mask(cross_attention_mask: torch.Tensor, num_vision_tokens: int,
-                                   kv_len: Optional[torch.Tensor] = None):
+                                   kv_len: Optional[torch.Tensor] = None, empty_rows: str = "all"):
     """Compact form of a Llama-3.2 cross-attention mask.
 
     `cross_attention_mask` is what the Mllama processor emits, [B, T, n_images,
@@ -161,11 +171,19 @@ def mask_from_cross_attention_mask(cross_attention_mask: torch.Tensor, num_visio
     (lv_xattn/attn.py:386-389).  When every row's visible keys form one
     contiguous range (the usual case: a token looks at the tiles of the most
     recent image) this returns `Mask(kv_len, kv_start, kv_end)` for the interval
-    kernels - 8 bytes per row instead of 4 bytes per (row, key); rows that see
-    nothing get an empty interval (O = 0, LSE = -inf, dQ = 0).  Returns None if
+    kernels - 8 bytes per row instead of 4 bytes per (row, key).  Returns None if
     some row has a gap (e.g. unused tile slots between two visible images): use
-    the dense bias then."""
+    the dense bias then.
+
+    A row that may look at no tile (text before the first image) follows
+    `empty_rows`: "all" (default) lets it see every key, which is what
+    `_prepare_cross_attention_mask` makes of it (it multiplies the additive mask
+    by full_text_row_masked_out_mask) and hence what the dense bias of the
+    reference holds; "none" gives it an empty interval (O = 0, LSE = -inf,
+    dQ = 0)."""
     from .ops import Mask
+    if empty_rows not in ("all", "none"):
+        raise ValueError("empty_rows must be 'all' or 'none'")
     B, T = cross_attention_mask.shape[:2]
     vis = cross_attention_mask.reshape(B, T, -1) != 0              # [B, T, n_images * n_tiles]
     n = vis.shape[-1]
@@ -176,7 +194,8 @@ def mask_from_cross_attention_mask(cross_attention_mask: torch.Tensor, num_visio
     count = vis.sum(-1)
     if not bool(((last - first + 1 == count) | ~any_vis).all()):
         return None
+    empty_end = n if empty_rows == "all" else 0
     start = torch.where(any_vis, first, torch.zeros_like(first)) * num_vision_tokens
-    end = torch.where(any_vis, last + 1, torch.zeros_like(last)) * num_vision_tokens
+    end = torch.where(any_vis, last + 1, torch.full_like(last, empty_end)) * num_vision_tokens
     return Mask(None if kv_len is None else kv_len.to(torch.int32), start.to(torch.int32).contiguous(),
                 end.to(torch.int32).contiguous())

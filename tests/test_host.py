@@ -84,14 +84,21 @@ def test_llama_cross_attention_mask_to_intervals():
     cam[0, 4:, 1, :] = 1            # tokens 4-5 see all four tiles of image 1
     cam[1, 2:, 0, :4] = 1           # sample 1: tokens 2.. see image 0 (4 tiles) ...
     cam[1, 5, 1, :1] = 1            # ... and token 5 also tile 0 of image 1 (adjacent: still one range)
-    m = mask_from_cross_attention_mask(cam, 5)
+    m = mask_from_cross_attention_mask(cam, 5, empty_rows="none")
     assert m is not None and m.kv_start.dtype == torch.int32
     assert m.kv_start.tolist() == [[0, 0, 0, 0, 20, 20], [0, 0, 0, 0, 0, 0]]
     assert m.kv_end.tolist() == [[0, 10, 10, 10, 40, 40], [0, 0, 20, 20, 20, 25]]
-    # the dense expansion transformers builds says the same
+    # the dense expansion says the same
     dense = cam.reshape(2, 6, 8).repeat_interleave(5, dim=-1).bool()
     k = torch.arange(40)
     assert torch.equal(dense, (k >= m.kv_start[..., None]) & (k < m.kv_end[..., None]))
+    # default: rows that may look at no tile see every key, which is what transformers' own
+    # mask preparation makes of them
+    from transformers.models.mllama.modeling_mllama import _prepare_cross_attention_mask
+    m = mask_from_cross_attention_mask(cam, 5)
+    assert m.kv_end.tolist() == [[40, 10, 10, 10, 40, 40], [40, 40, 20, 20, 20, 25]]
+    hf_mask, _ = _prepare_cross_attention_mask(cam.float(), 5, torch.float32)       # [B, 1, T, keys], 0 = visible
+    assert torch.equal(hf_mask[:, 0] == 0, (k >= m.kv_start[..., None]) & (k < m.kv_end[..., None]))
     # a gap (image 0 with 2 of 4 tiles, then image 1) has no interval form
     cam[0, 5, 0, :2] = 1
     assert mask_from_cross_attention_mask(cam, 5) is None
