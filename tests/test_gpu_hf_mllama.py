@@ -93,12 +93,13 @@ def test_mllama_cross_attention_layer_matches_eager(variant, dtype):
         assert rel(gp_n[n], gp_r[n]) < 3e-2, n
 
 
-@pytest.mark.parametrize("variant", ["interface", "recompute"])
+@pytest.mark.parametrize("variant", ["interface", "recompute", "recompute_intervals"])
 def test_tiny_mllama_text_model_matches_eager(variant):
     """A four-layer MllamaForCausalLM (two self-attention, two cross-attention decoder layers,
     random weights) end to end.  Truth is the model in fp32 with transformers' eager attention;
     the bf16 model with the "lv_xattn" implementation (interface hook, or the patched recompute
-    forward on both cross-attention layers) must come as close to it as the bf16 model with
+    forward on both cross-attention layers, there also with the mask handed through the model's
+    keyword arguments as per-row key intervals) must come as close to it as the bf16 model with
     eager attention does (within a factor 2), in the logits and in every gradient."""
     pytest.importorskip("transformers")
     from transformers.models.mllama import modeling_mllama as m
@@ -125,7 +126,7 @@ def test_tiny_mllama_text_model_matches_eager(variant):
     ref.load_state_dict(truth.state_dict())          # the same bf16-rounded weights in both bf16 models
     new.load_state_dict(ref.state_dict())
     truth.load_state_dict(ref.state_dict())          # and those exact values in the fp32 one
-    if variant == "recompute":
+    if variant != "interface":
         assert hf_mllama.patch_cross_attention_forward(new) == 2
 
     g = torch.Generator().manual_seed(21)
@@ -144,8 +145,16 @@ def test_tiny_mllama_text_model_matches_eager(variant):
         full = allowed.any(-1).to(dtype)[..., None]                   # [B, 1, Lq, 1]
         cmask = torch.zeros(B, 1, Lq, Lkv, dtype=dtype, device=DEV).masked_fill(~allowed, torch.finfo(dtype).min) * full
         v = vis.to(dtype).clone().requires_grad_()
+        extra = {}
+        if model is new and variant == "recompute_intervals":
+            # the processor's form of the same mask: [B, T, images, tiles], one image of two tiles
+            cam = torch.zeros(B, Lq, 1, 2, dtype=torch.int64)
+            cam[0, 9:] = 1
+            cam[1, :, 0, 0] = 1
+            extra["lvx_mask"] = hf_mllama.mask_from_cross_attention_mask(cam.to(DEV), 800, kv_len=torch.tensor([Lkv, Lkv]))
+            cmask = torch.zeros_like(cmask)      # the dense mask says nothing: only the intervals can get it right
         out = model(input_ids=ids, cross_attention_states=v, cross_attention_mask=cmask,
-                    full_text_row_masked_out_mask=full, use_cache=False)
+                    full_text_row_masked_out_mask=full, use_cache=False, **extra)
         (out.logits.float() * go.float()).sum().backward()
         torch.cuda.synchronize()
         grads = {n: p.grad.float() for n, p in model.named_parameters() if p.grad is not None}
