@@ -180,3 +180,66 @@ def test_tiny_mllama_text_model_matches_eager(variant):
         if e_new > max(2 * e_ref, floor):
             bad.append((n, e_new, e_ref))
     assert not bad, bad
+
+
+@pytest.mark.parametrize("variant", ["interface", "recompute"])
+def test_tiny_mllama_prefill_then_decode_with_cache(variant):
+    """Inference with a K/V cache: a prefill over the prompt (cross-attention states given),
+    then two single-token steps that read the cached cross-attention K/V (no states given).
+    Logits of every step against the same bf16 model with eager attention."""
+    pytest.importorskip("transformers")
+    from transformers import DynamicCache
+    from transformers.models.mllama import modeling_mllama as m
+    from transformers.models.mllama.configuration_mllama import MllamaTextConfig
+    from lv_xattn import _lib, hf_mllama
+    _lib.load()
+    name = hf_mllama.register()
+
+    def build(impl):
+        cfg = MllamaTextConfig(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, num_hidden_layers=4,
+                               intermediate_size=256, cross_attention_layers=[1, 3], vocab_size=128,
+                               bos_token_id=1, eos_token_id=2, pad_token_id=0, max_position_embeddings=512)
+        cfg._attn_implementation = impl
+        torch.manual_seed(9)
+        model = m.MllamaForCausalLM(cfg)
+        with torch.no_grad():
+            for layer in model.model.layers:
+                if hasattr(layer, "cross_attn_attn_gate"):
+                    layer.cross_attn_attn_gate.fill_(0.7)
+                    layer.cross_attn_mlp_gate.fill_(0.4)
+        return model.to(device=DEV, dtype=torch.bfloat16).eval()
+
+    ref, new = build("eager"), build(name)
+    new.load_state_dict(ref.state_dict())
+    if variant == "recompute":
+        assert hf_mllama.patch_cross_attention_forward(new) == 2
+
+    g = torch.Generator().manual_seed(33)
+    B, Lq, Lkv, steps = 2, 70, 1601, 2
+    ids = torch.randint(3, 128, (B, Lq + steps), generator=g).to(DEV)
+    vis = torch.randn(B, Lkv, 1024, generator=g).bfloat16().to(DEV)
+    allowed = torch.ones(B, 1, Lq + steps, Lkv, dtype=torch.bool)
+    allowed[0, :, :5, :] = False
+    allowed[1, :, :, 800:] = False
+    full = allowed.any(-1).to(torch.bfloat16)[..., None].to(DEV)
+    cmask = (torch.zeros(B, 1, Lq + steps, Lkv, dtype=torch.bfloat16)
+             .masked_fill(~allowed, torch.finfo(torch.bfloat16).min).to(DEV)) * full
+
+    def rel(a, b):
+        return ((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-12)).item()
+
+    outs = []
+    with torch.no_grad():
+        for model in (ref, new):
+            cache = DynamicCache(config=model.config)
+            lo = [model(input_ids=ids[:, :Lq], cross_attention_states=vis, cross_attention_mask=cmask[:, :, :Lq],
+                        full_text_row_masked_out_mask=full[:, :, :Lq], past_key_values=cache, use_cache=True).logits]
+            for t in range(Lq, Lq + steps):
+                lo.append(model(input_ids=ids[:, t:t + 1], cross_attention_mask=cmask[:, :, t:t + 1],
+                                full_text_row_masked_out_mask=full[:, :, t:t + 1], past_key_values=cache,
+                                use_cache=True).logits)
+            torch.cuda.synchronize()
+            outs.append(lo)
+    for step, (a, b) in enumerate(zip(outs[1], outs[0])):
+        assert a.shape == b.shape and torch.isfinite(a).all()
+        assert rel(a, b) < 3e-2, (step, rel(a, b))
