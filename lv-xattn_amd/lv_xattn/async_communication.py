@@ -3,8 +3,8 @@
 
 On one MI355X there is no neighbour to exchange query blocks with: the P
 "ranks" of the sequence-parallel group become P rounds of an on-device loop.
-Only the three names callers import survive (lv_xattn/__init__.py:1-2 of the
-reference); they keep their call signatures and do the little that is left to
+The names callers import survive (lv_xattn/__init__.py:1-2 of the reference,
+plus the size / rank / destroy helpers); they keep their call signatures and do the little that is left to
 do: pick the device, remember P, drop cached workspaces.
 """
 from __future__ import annotations
@@ -59,6 +59,14 @@ def get_sequence_parallel_size() -> int:
 
 def get_sequence_parallel_rank() -> int:
     return 0
+
+
+def destroy_sequence_parallel() -> None:
+    """Reference: drops the process group (async_communication.py:205-208).
+    Here: back to one round, cached workspaces freed."""
+    global _ROUNDS, _INITIALISED
+    _ROUNDS, _INITIALISED = 1, False
+    _WORKSPACES.clear()
 
 
 def reset_global_memory_buffer(*_ignored) -> None:

@@ -33,7 +33,10 @@ def test_round_group_shim(monkeypatch):
     assert lv_xattn.get_sequence_parallel_group().size() == 4
     with pytest.raises(ValueError):
         ac.initialize_distributed(0)
-    ac.initialize_distributed(1)
+    ac.initialize_distributed(3)
+    assert ac.get_sequence_parallel_size() == 3 and ac.get_sequence_parallel_rank() == 0
+    ac.destroy_sequence_parallel()
+    assert ac.get_sequence_parallel_size() == 1
 
 
 def test_workspace_cache_and_reset():
