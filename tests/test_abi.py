@@ -135,3 +135,54 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liblvx.so")
     with pytest.raises(_lib.LvxError, match="no CPU fallback"):
         _lib.load()
+
+
+C_CALLER = r"""
+#include <dlfcn.h>
+#include <stdio.h>
+#include <string.h>
+#include "lvx.h"
+
+int main(int argc, char** argv) {
+    void* h = dlopen(argv[1], RTLD_NOW | RTLD_LOCAL);
+    if (!h) { fprintf(stderr, "%s\n", dlerror()); return 2; }
+    int (*version)(void) = (int (*)(void))dlsym(h, "lvx_version");
+    const char* (*strerr)(int) = (const char* (*)(int))dlsym(h, "lvx_strerror");
+    int (*fwd)(const lvx_attn_shape*, const lvx_tensor*, const lvx_tensor*, const lvx_tensor*, const lvx_tensor*,
+               float*, int32_t, int32_t, int32_t, void*, size_t, void*) =
+        (int (*)(const lvx_attn_shape*, const lvx_tensor*, const lvx_tensor*, const lvx_tensor*, const lvx_tensor*,
+                 float*, int32_t, int32_t, int32_t, void*, size_t, void*))dlsym(h, "lvx_fwd");
+    size_t (*ws)(const lvx_attn_shape*, int32_t, int32_t) =
+        (size_t (*)(const lvx_attn_shape*, int32_t, int32_t))dlsym(h, "lvx_fwd_workspace_bytes");
+    if (!version || !strerr || !fwd || !ws) return 3;
+    lvx_attn_shape s;
+    memset(&s, 0, sizeof s);
+    s.B = 1; s.Hq = 8; s.Hkv = 2; s.D = 64; s.Lq = 64; s.Lkv = 256; s.dtype = LVX_BF16; s.scale = 0.125f;
+    lvx_tensor t = {(void*)0x1000, 8 * 64 * 128, 64 * 128, 128};
+    int rc = fwd(&s, &t, &t, &t, &t, (float*)0x2000, 0, 64, 1, NULL, 0, NULL);   /* rejected on the host: D != 128 */
+    s.D = 128;
+    printf("%d|%d|%s|%zu\n", version(), rc, strerr(rc), ws(&s, 64, 4));
+    return 0;
+}
+"""
+
+
+def test_plain_c_caller_compiles_against_the_header_and_calls_the_library(lib, tmp_path):
+    """The boundary is a C ABI: a C99 translation unit including lvx.h builds with gcc, loads
+    the library and gets the host-side argument check (no GPU involved)."""
+    import shutil
+    import subprocess
+    from lv_xattn import _lib
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "caller.c"
+    src.write_text(C_CALLER)
+    exe = tmp_path / "caller"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe), "-ldl"],
+                   check=True, capture_output=True, text=True)
+    r = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    version, rc, msg, ws = r.stdout.strip().split("|")
+    assert int(version) == 100 and int(rc) == -4 and msg == "head_dim must be 128"
+    assert int(ws) == 4 * 8 * 64 * (128 * 2 + 4)
