@@ -137,6 +137,20 @@ def test_random_shape_forward_backward_fp16(lvx, seed):
               dtype=torch.float16, sigma=0.5)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shape_many_heads_and_samples(lvx, seed):
+    # more samples and heads than the other cases: the block -> (sample, head group, tile)
+    # decoding of every kernel, head groupings of 1, 4, 8 and 32
+    rng = random.Random(12000 + seed)
+    g = torch.Generator().manual_seed(13000 + seed)
+    B = rng.choice([4, 5, 8, 11])
+    Hq, Hkv = [(32, 8), (16, 16), (24, 3), (64, 8), (32, 1), (20, 5)][seed]
+    Lq, Lkv = rng.randint(1, 300), rng.randint(1, 700)
+    mask_kind = ["none", "kv_len", "intervals"][seed % 3]
+    _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rng.choice([1, 2, 5]), seed % 2 == 0, mask_kind, rng, g, strided=seed == 4,
+              dtype=[torch.bfloat16, torch.float16][seed % 2], sigma=[1.0, 0.5][seed % 2])
+
+
 @pytest.mark.parametrize("batched", [True, False])
 def test_more_than_four_runs_of_live_row_groups(lvx, batched):
     # 10 groups of 256 rows; group i sees only token block i % 2, so each of the two token
