@@ -243,3 +243,60 @@ def test_tiny_mllama_prefill_then_decode_with_cache(variant):
     for step, (a, b) in enumerate(zip(outs[1], outs[0])):
         assert a.shape == b.shape and torch.isfinite(a).all()
         assert rel(a, b) < 3e-2, (step, rel(a, b))
+
+
+def test_tiny_mllama_left_padded_batch():
+    """A left-padded batch: the self-attention layers, which reach the hook under the same
+    implementation name, must see transformers' causal + padding mask (a custom name gets none
+    unless a mask builder is registered with it).  Logits at the real tokens against the eager
+    model, with transformers' own SDPA model as the yardstick."""
+    pytest.importorskip("transformers")
+    from transformers.models.mllama import modeling_mllama as m
+    from transformers.models.mllama.configuration_mllama import MllamaTextConfig
+    from lv_xattn import _lib, hf_mllama
+    _lib.load()
+    name = hf_mllama.register()
+
+    def build(impl):
+        cfg = MllamaTextConfig(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, num_hidden_layers=4,
+                               intermediate_size=256, cross_attention_layers=[1, 3], vocab_size=128,
+                               bos_token_id=1, eos_token_id=2, pad_token_id=0, max_position_embeddings=512)
+        cfg._attn_implementation = impl
+        torch.manual_seed(5)
+        model = m.MllamaForCausalLM(cfg)
+        with torch.no_grad():
+            for layer in model.model.layers:
+                if hasattr(layer, "cross_attn_attn_gate"):
+                    layer.cross_attn_attn_gate.fill_(0.7)
+                    layer.cross_attn_mlp_gate.fill_(0.4)
+        return model.to(device=DEV, dtype=torch.bfloat16).eval()
+
+    ref, new, sdpa = build("eager"), build(name), build("sdpa")
+    new.load_state_dict(ref.state_dict())
+    sdpa.load_state_dict(ref.state_dict())
+    g = torch.Generator().manual_seed(3)
+    B, Lq, Lkv, pad = 2, 90, 1601, 25
+    ids = torch.randint(3, 128, (B, Lq), generator=g)
+    ids[1, :pad] = 0
+    am = torch.ones(B, Lq, dtype=torch.long)
+    am[1, :pad] = 0
+    vis = torch.randn(B, Lkv, 1024, generator=g).bfloat16().to(DEV)
+    allowed = torch.ones(B, 1, Lq, Lkv, dtype=torch.bool)
+    allowed[0, :, :9] = False
+    allowed[1, :, :, 800:] = False
+    full = allowed.any(-1).to(torch.bfloat16)[..., None].to(DEV)
+    cmask = torch.zeros(B, 1, Lq, Lkv, dtype=torch.bfloat16).masked_fill(~allowed, torch.finfo(torch.bfloat16).min).to(DEV) * full
+    outs = []
+    with torch.no_grad():
+        for model in (ref, new, sdpa):
+            outs.append(model(input_ids=ids.to(DEV), attention_mask=am.to(DEV), cross_attention_states=vis,
+                              cross_attention_mask=cmask, full_text_row_masked_out_mask=full,
+                              use_cache=False).logits.float())
+    torch.cuda.synchronize()
+    valid = am.bool().to(DEV)
+
+    def rel(a, b):
+        return ((a - b)[valid].norm() / b[valid].norm()).item()
+
+    assert torch.isfinite(outs[1][valid]).all()
+    assert rel(outs[1], outs[0]) <= max(2 * rel(outs[2], outs[0]), 1e-2), (rel(outs[1], outs[0]), rel(outs[2], outs[0]))
