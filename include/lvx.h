@@ -97,6 +97,24 @@ int lvx_fwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* 
 size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* shape, int32_t row_count, int32_t kv_splits);
 
 /*
+ * lvx_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  The key-split partials go to an array inside the library
+ * (LVX_NOALLOC_SCRATCH_BYTES of device memory per GPU, held until the process ends) instead
+ * of a caller's workspace; the call allocates and frees nothing.  Same arguments, results
+ * and return codes as lvx_fwd otherwise; LVX_ERR_WORKSPACE when
+ * lvx_fwd_workspace_bytes(shape, row_count, kv_splits) exceeds the array.  The array belongs
+ * to the device that is current when the call is made, which must be the stream's device.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams,
+ * two threads) race; calls queued on one stream do not.
+ */
+#define LVX_NOALLOC_SCRATCH_BYTES (16u << 20)
+int lvx_fwd_noalloc(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,
+                    const lvx_tensor* v, const lvx_tensor* o, float* lse,
+                    int32_t row_begin, int32_t row_count, int32_t kv_splits, void* stream);
+size_t lvx_noalloc_scratch_bytes(void);
+
+/*
  * Rescale-merge: folds a partial (o_part, l_part) over one key set into the
  * travelling accumulator (o_acc, l_acc) of the same rows, in place:
  *   L' = ln(e^La + e^Lb),  O' = Oa e^(La-L') + Ob e^(Lb-L').

@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <mutex>
 
 using namespace lvx;
 
@@ -58,6 +59,37 @@ constexpr int MAX_SPLITS = 16;
 }  // namespace
 
 static void fill_grid(GemmParams& g, int M, int N, int nprob, int nbatch);
+
+// Device memory of lvx_fwd_noalloc: the key-split partials live in this file-scope array
+// instead of a caller's workspace.  Every GPU the library runs on holds its own copy at its
+// own address until the process ends; the address is asked for once per device.
+constexpr size_t NOALLOC_SCRATCH_BYTES = LVX_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES];      // per device: where that device keeps `scratch`
+
+// The device address of `scratch` on the current device (the array's name is a host-side
+// stand-in, not an address a kernel can use).
+int scratch_on_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= MAX_DEVICES) return LVX_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!ptr) return LVX_ERR_UNSUPPORTED;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return LVX_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -166,6 +198,21 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     m.B = s->B; m.Hq = s->Hq; m.Lq = s->Lq;
     m.row_begin = row_begin; m.row_end = row_begin + row_count;
     return static_cast<int>(launch_merge(m, st));
+}
+
+size_t lvx_noalloc_scratch_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+int lvx_fwd_noalloc(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+                    const lvx_tensor* o, float* lse, int32_t row_begin, int32_t row_count, int32_t kv_splits,
+                    void* stream) {
+    // argument errors first, as lvx_fwd reports them
+    LVX_TRY(check_shape(s));
+    if (kv_splits < 1 || kv_splits > MAX_SPLITS) return LVX_ERR_SHAPE;
+    if (row_count > 0 && lvx_fwd_workspace_bytes(s, row_count, kv_splits) > NOALLOC_SCRATCH_BYTES)
+        return LVX_ERR_WORKSPACE;     // the partials of this call do not fit the library's own array
+    void* ws = nullptr;
+    LVX_TRY(scratch_on_current_device(&ws));
+    return lvx_fwd(s, q, k, v, o, lse, row_begin, row_count, kv_splits, ws, NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int lvx_merge(const lvx_attn_shape* s, const lvx_tensor* o_acc, float* l_acc, const lvx_tensor* o_part,

@@ -94,6 +94,24 @@ def fwd(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask
     check(rc, "lvx_fwd")
 
 
+def noalloc_scratch_bytes() -> int:
+    """Size of the library's own array that fwd_noalloc keeps its key-split partials in."""
+    return int(load().lvx_noalloc_scratch_bytes())
+
+
+def fwd_noalloc(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask] = None,
+                kv_splits: int = 1, bias: Optional[torch.Tensor] = None) -> None:
+    """`fwd` without a workspace argument and without any allocation: the key-split
+    partials go to an array inside the library (one per GPU, shared by all calls on it)."""
+    s = _shape(q, k, scale, mask, bias)
+    if row_count is None:
+        row_count = q.shape[2] - row_begin
+    _check_lse(lse, q)
+    rc = load().lvx_fwd_noalloc(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(o)),
+                                lse.data_ptr(), row_begin, row_count, kv_splits, stream_ptr())
+    check(rc, "lvx_fwd_noalloc")
+
+
 def merge(o_acc, l_acc, o_part, l_part, row_begin=0, row_count=None) -> None:
     """(o_acc, l_acc) <- LSE-merge of itself with (o_part, l_part), in place."""
     B, Hq, Lq, D = o_acc.shape
