@@ -25,9 +25,20 @@ for p in (ROOT, os.path.join(ROOT, "lv-xattn_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
-# HBM bytes moved by one lvx_bwd call at cfg2 (zero + dK/dV kernel + 2 casts + dQ GEMM), from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 1 GiB copy (profiles/cfg2_bwd_hbm_traffic.md)
-BWD_TRAFFIC_BYTES = {"cfg2": 4.41e9}
+
+
+def bwd_traffic_bytes(name):
+    """HBM bytes moved by one lvx_bwd call (metadata + dK/dV kernel + 2 casts + dQ GEMM) as
+    the counter summary of that workload states them (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    runs scaled by a 1 GiB copy): the `traffic_bytes_per_call:` line of
+    profiles/<name>_bwd_hbm_traffic.md.  None when there is no such summary."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{name}_bwd_hbm_traffic.md")
+    try:
+        m = re.search(r"^traffic_bytes_per_call:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    except OSError:
+        return None
+    return float(m.group(1)) if m else None
 
 
 def flops(w, n_pairs):
@@ -220,6 +231,89 @@ def run_only(layer, which, n, torch):
                       "avg_launch_ms": round(e0.elapsed_time(e1) / n, 5)}))
 
 
+def hbm_bytes(w):
+    """Algorithmic HBM bytes of one step: every operand read once and every result written once
+    per operator (projection twice, forward, merge, preprocess, backward, dX_vis); the backward's
+    dS^T workspace is not part of it."""
+    e = 2                                            # bytes per element
+    q = w.B * w.Hq * w.Lq * w.D * e
+    kv = 2 * w.B * w.Hkv * w.Lkv * w.D * e
+    lse = w.B * w.Hq * w.Lq * 4
+    total = (q + kv) + (q + lse)                     # forward: Q, K, V in; O, LSE out
+    total += 3 * q + 3 * lse                         # merge: two O + two LSE in, O + LSE out
+    total += 2 * q + lse                             # preprocess: O, dO in; delta out
+    total += (2 * q + kv + 2 * lse) + (q + kv)       # backward: Q, dO, K, V, LSE, delta in; dQ, dK, dV out
+    if w.Dm:
+        x = w.B * w.Lkv * w.Dm * e
+        wt = 2 * w.Dm * w.Hkv * w.D * e
+        total += 2 * (x + wt + kv) + (kv + wt + x)   # K/V projection twice, dX_vis
+    return total
+
+
+def other_workload(name, torch, dev, steps=10, warmup=5):
+    """One more workload under the same clock, in both modes: ms per step, TFLOP/s on the pairs
+    its mask leaves alive, fraction of the MFMA peak, algorithmic HBM GB/s, and the forward and
+    backward operators on their own."""
+    from oracle import lvx_oracle as orc
+    w = orc.make_inputs(orc.workload(name))
+    npairs = orc.n_pairs(w)
+    f = flops(w, npairs)
+    fwd_only = name == "cfg1"
+    layer = Layer(w, "batched", dev)
+    rec = {"workload": f"{w.name}: B{w.B} Hq{w.Hq} Hkv{w.Hkv} D{w.D} Lq{w.Lq}={w.rounds}x{-(-w.Lq // w.rounds)} "
+                       f"Lkv{w.Lkv} Dm{w.Dm}" + (" masked ragged" if layer.mask is not None else "")
+                       + (" (forward + merge only)" if fwd_only else "")}
+    if fwd_only:
+        k, v = layer.project()
+        step_flops = f["fwd"]
+        fns = {"batched": lambda: layer.forward(k, v)}
+        other = Layer(w, "rounds", dev)
+        fns["rounds"] = lambda: other.forward(k, v)
+    else:
+        step_flops = f["fwd"] + f["bwd"] + 3 * f["proj"]
+        other = Layer(w, "rounds", dev)
+        fns = {"batched": layer.step, "rounds": other.step}
+    rec["flops_per_step"] = step_flops
+    for mode, fn in fns.items():
+        ms = time_gpu(fn, steps, warmup, torch)
+        rec[mode] = {"ms_per_step": round(ms, 4), "tflops": round(step_flops / ms / 1e9, 2),
+                     "frac_bf16_mfma_peak": round(step_flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        if not fwd_only:
+            rec[mode]["hbm_algorithmic_gbs"] = round(hbm_bytes(w) / ms / 1e6, 1)
+    if not fwd_only:
+        ops = layer.ops
+        k, v = layer.project()
+        o, L = layer.forward(k, v)
+        B, Hq, Lq, D = layer.q.shape
+        Hkv, Lkv = k.shape[1], k.shape[2]
+        o_p, l_p, delta = torch.empty_like(o), torch.empty_like(L), torch.empty_like(L)
+        ops.bwd_preprocess(o, layer.do, delta)
+        dq = torch.empty_like(layer.q)
+        bws = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, layer.mask), dtype=torch.uint8, device=dev)
+        dk = torch.empty(B, Lkv, Hkv, D, dtype=w.dtype, device=dev).transpose(1, 2)
+        dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
+        ms = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=layer.mask), steps, warmup, torch)
+        rec["lvx_fwd"] = {"ms": round(ms, 4), "tflops": round(f["fwd"] / ms / 1e9, 1)}
+        ms = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask,
+                                      workspace=bws), steps, warmup, torch)
+        rec["lvx_bwd"] = {"ms": round(ms, 4), "tflops": round(f["bwd"] / ms / 1e9, 1)}
+        merge_bytes = (3 * D * 2 + 3 * 4) * B * Hq * Lq
+        ms = time_gpu(lambda: ops.merge(o_p, l_p, o, L), steps, warmup, torch)
+        rec["lvx_merge"] = {"ms": round(ms, 4), "gbs": round(merge_bytes / ms / 1e6, 1),
+                            "frac_hbm": round(merge_bytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        if layer.has_proj:
+            ms = time_gpu(layer.project, steps, warmup, torch)
+            rec["lvx_kv_proj"] = {"ms": round(ms, 4), "tflops": round(f["proj"] / ms / 1e9, 1)}
+            ms = time_gpu(lambda: ops.dx_vis(dk, dv, layer.wk, layer.wv), steps, warmup, torch)
+            rec["lvx_dx_vis"] = {"ms": round(ms, 4), "tflops": round(f["proj"] / ms / 1e9, 1)}
+    del layer, other
+    layer = other = None
+    from lv_xattn import reset_global_memory_buffer
+    reset_global_memory_buffer()
+    torch.cuda.empty_cache()
+    return rec
+
+
 def cpu_baseline(w, budget_rounds=8):
     """The oracle (the reference's PyTorch math restated) timed on this host's
     cores on a bounded sample: the first `budget_rounds` query blocks, forward
@@ -272,6 +366,7 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-others", action="store_true", help="skip the sub-records of cfg1, cfg3 and cfg4")
     ap.add_argument("--only", choices=["fwd", "bwd", "kv_proj", "dx_vis", "copy"],
                     help="launch just this operator --steps times (for rocprofv3 counter runs); "
                          "'copy' is a 1 GiB device copy that calibrates FETCH_SIZE / WRITE_SIZE")
@@ -328,12 +423,19 @@ def main():
         out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel (incl. scratch zero-fill) + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
                            "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
-                           "traffic": BWD_TRAFFIC_BYTES.get(w.name) if a.mode == "batched" else None,
+                           "traffic": bwd_traffic_bytes(w.name) if a.mode == "batched" else None,
                            "flops_per_launch": f["bwd"], "avg_launch_ms": dom["ms"]}
         other = Layer(w, "rounds" if a.mode == "batched" else "batched", dev)
         ms2 = time_gpu(other.step, max(3, a.steps // 2), 2, torch)
         out["config"]["other_mode"] = {"mode": other.mode, "ms_per_step": round(ms2, 4),
                                        "tflops": round(step_flops / ms2 / 1e9, 2)}
+    if not a.no_others and w.name == "cfg2" and a.dtype == "bf16":
+        # the other GPU configurations under the same clock (the headline stays cfg2)
+        del layer
+        from lv_xattn import reset_global_memory_buffer
+        reset_global_memory_buffer()
+        torch.cuda.empty_cache()
+        out["config"]["other_workloads"] = {n: other_workload(n, torch, dev) for n in ("cfg1", "cfg3", "cfg4")}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, min(8, w.rounds))
     print(json.dumps(out))
