@@ -62,8 +62,9 @@ typedef struct lvx_attn_shape {
      * reference's bias_func returns, lv_xattn/attn.py:386-389, 238-241), or NULL.  Element
      * (b, h, row, key) is at bias[b*bias_stride_b + h*bias_stride_h + row*bias_stride_r + key];
      * bias_stride_h = 0 broadcasts over heads.  -inf entries mask.  No gradient is formed
-     * for it (the reference forms none).  Rows are read in groups of 4 keys, so
-     * bias_stride_r must be at least Lkv rounded up to a multiple of 4 (pad the rows).
+     * for it (the reference forms none).  Rows are read in groups of 4 keys with 16-byte
+     * loads: bias must be 16-byte aligned, the three strides multiples of 4 (LVX_ERR_ALIGN
+     * otherwise), and bias_stride_r at least Lkv rounded up to a multiple of 4 (pad the rows).
      * Mask with -inf or a moderate negative (e.g. -30000), not with -FLT_MAX-sized values:
      * the backward subtracts the row's LSE from score + bias in fp32. */
     const float* bias;

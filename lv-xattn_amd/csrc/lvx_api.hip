@@ -30,8 +30,10 @@ int check_shape(const lvx_attn_shape* s) {
     if (!(s->scale > 0.f) || !std::isfinite(s->scale)) return LVX_ERR_SCALE;
     if ((s->kv_start == nullptr) != (s->kv_end == nullptr)) return LVX_ERR_NULL;
     if (s->bias) {
-        if (reinterpret_cast<uintptr_t>(s->bias) & 3) return LVX_ERR_ALIGN;
-        // rows are read in groups of 4 keys: a row must be readable up to Lkv rounded up to 4
+        // rows are read in groups of 4 keys with 16-byte loads: every row must start on a
+        // 16-byte boundary and be readable up to Lkv rounded up to 4
+        if (reinterpret_cast<uintptr_t>(s->bias) & 15) return LVX_ERR_ALIGN;
+        if ((s->bias_stride_r | s->bias_stride_h | s->bias_stride_b) & 3) return LVX_ERR_ALIGN;
         if (s->bias_stride_r < (s->Lkv + 3) / 4 * 4) return LVX_ERR_SHAPE;
     }
     return LVX_OK;

@@ -543,22 +543,21 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
 namespace {
 template <bool F16>
-void launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
+hipError_t launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) hipLaunchKernelGGL((bwd_kernel<true, true, F16>), dim3(grid), dim3(NT), 0, st, p);
-        else hipLaunchKernelGGL((bwd_kernel<false, true, F16>), dim3(grid), dim3(NT), 0, st, p);
+        if (masked) return launch1((bwd_kernel<true, true, F16>), dim3(grid), dim3(NT), st, p);
+        else return launch1((bwd_kernel<false, true, F16>), dim3(grid), dim3(NT), st, p);
     } else {
-        if (masked) hipLaunchKernelGGL((bwd_kernel<true, false, F16>), dim3(grid), dim3(NT), 0, st, p);
-        else hipLaunchKernelGGL((bwd_kernel<false, false, F16>), dim3(grid), dim3(NT), 0, st, p);
+        if (masked) return launch1((bwd_kernel<true, false, F16>), dim3(grid), dim3(NT), st, p);
+        else return launch1((bwd_kernel<false, false, F16>), dim3(grid), dim3(NT), st, p);
     }
 }
 }  // namespace
 
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
-    if (p.f16) launch_bwd_t<true>(p, masked, st);
-    else launch_bwd_t<false>(p, masked, st);
-    return hipGetLastError();
+    if (p.f16) return launch_bwd_t<true>(p, masked, st);
+    return launch_bwd_t<false>(p, masked, st);
 }
 
 }  // namespace lvx

@@ -325,22 +325,21 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
 namespace {
 template <bool F16>
-void launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
+hipError_t launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) hipLaunchKernelGGL((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), 0, st, p);
+        if (masked) return launch1((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), st, p);
+        else return launch1((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), st, p);
     } else {
-        if (masked) hipLaunchKernelGGL((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), 0, st, p);
+        if (masked) return launch1((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), st, p);
+        else return launch1((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), st, p);
     }
 }
 }  // namespace
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
-    if (p.f16) launch_fwd_t<true>(p, masked, st);
-    else launch_fwd_t<false>(p, masked, st);
-    return hipGetLastError();
+    if (p.f16) return launch_fwd_t<true>(p, masked, st);
+    return launch_fwd_t<false>(p, masked, st);
 }
 
 }  // namespace lvx

@@ -351,15 +351,15 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
 }
 
 template <int GM, int GN, int WM, int WN, int NS, bool F16>
-void launch_cfg_t(const GemmParams& p, int grid, bool a_mcontig, bool b_ncontig, hipStream_t st) {
+hipError_t launch_cfg_t(const GemmParams& p, int grid, bool a_mcontig, bool b_ncontig, hipStream_t st) {
     if (!a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+        return launch1((gemm_kernel<false, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), st, p);
     else if (!a_mcontig && b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<false, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+        return launch1((gemm_kernel<false, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), st, p);
     else if (a_mcontig && !b_ncontig)
-        hipLaunchKernelGGL((gemm_kernel<true, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+        return launch1((gemm_kernel<true, false, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), st, p);
     else
-        hipLaunchKernelGGL((gemm_kernel<true, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), 0, st, p);
+        return launch1((gemm_kernel<true, true, GM, GN, WM, WN, NS, F16>), dim3(grid), dim3(512), st, p);
 }
 
 template <int GM, int GN, int WM, int WN, int NS>
@@ -369,9 +369,8 @@ hipError_t launch_cfg(GemmParams p, bool a_mcontig, bool b_ncontig, hipStream_t 
     p.tiles_n = (p.N + TN - 1) / TN;
     p.total_wg = p.nprob * p.nbatch * p.tiles_m * p.tiles_n * (p.k_splits > 1 ? p.k_splits : 1);
     const int grid = ((p.total_wg + 7) / 8) * 8;
-    if (p.f16) launch_cfg_t<GM, GN, WM, WN, NS, true>(p, grid, a_mcontig, b_ncontig, st);
-    else launch_cfg_t<GM, GN, WM, WN, NS, false>(p, grid, a_mcontig, b_ncontig, st);
-    return hipGetLastError();
+    if (p.f16) return launch_cfg_t<GM, GN, WM, WN, NS, true>(p, grid, a_mcontig, b_ncontig, st);
+    return launch_cfg_t<GM, GN, WM, WN, NS, false>(p, grid, a_mcontig, b_ncontig, st);
 }
 
 }  // namespace

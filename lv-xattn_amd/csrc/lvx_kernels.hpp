@@ -6,6 +6,15 @@
 
 namespace lvx {
 
+// Queues kernel(p) and returns that launch's own error code.  The thread's sticky "last error"
+// (which may hold an unrelated component's earlier failure) is neither read nor cleared.
+template <typename P>
+inline hipError_t launch1(void (*kernel)(P), dim3 grid, dim3 block, hipStream_t st, const P& p) {
+    P arg = p;
+    void* args[] = {&arg};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, args, 0, st);
+}
+
 struct Strides3 {
     int64_t b, h, s;
 };

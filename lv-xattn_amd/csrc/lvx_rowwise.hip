@@ -69,8 +69,11 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
         float f[8];
         unpack8<E>(*reinterpret_cast<const u32x4*>(oa), f);
         const float w = wa * inv;
+        // an accumulator with weight 0 (L = -inf: nothing folded in yet) may hold anything
+        if (w > 0.f) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = f[j] * w;
+            for (int j = 0; j < 8; ++j) out[j] = f[j] * w;
+        }
     }
     const uint16_t* op = p.o_part + b * p.op.b + h * p.op.h + (int64_t)row * p.op.s + chunk * 8;
 #pragma unroll
@@ -305,17 +308,15 @@ inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    if (p.f16) hipLaunchKernelGGL(merge_kernel<true>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(merge_kernel<false>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
-    return hipGetLastError();
+    if (p.f16) return launch1(merge_kernel<true>, dim3(blocks_for(rows)), dim3(256), st, p);
+    else return launch1(merge_kernel<false>, dim3(blocks_for(rows)), dim3(256), st, p);
 }
 
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    if (p.f16) hipLaunchKernelGGL(preprocess_kernel<true>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(preprocess_kernel<false>, dim3(blocks_for(rows)), dim3(256), 0, st, p);
-    return hipGetLastError();
+    if (p.f16) return launch1(preprocess_kernel<true>, dim3(blocks_for(rows)), dim3(256), st, p);
+    else return launch1(preprocess_kernel<false>, dim3(blocks_for(rows)), dim3(256), st, p);
 }
 
 hipError_t launch_bwd_meta(const MetaParams& p0, hipStream_t st) {
@@ -325,26 +326,22 @@ hipError_t launch_bwd_meta(const MetaParams& p0, hipStream_t st) {
     if (n == 0 && z == 0) return hipSuccess;
     p.meta_blocks = (int)((n + 255) / 256);
     const int zero_blocks = (int)std::min<int64_t>((z + 255) / 256, 2048);
-    hipLaunchKernelGGL(bwd_meta_kernel, dim3((unsigned)(p.meta_blocks + zero_blocks)), dim3(256), 0, st, p);
-    return hipGetLastError();
+    return launch1(bwd_meta_kernel, dim3((unsigned)(p.meta_blocks + zero_blocks)), dim3(256), st, p);
 }
 
 hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st) {
     if (p.B <= 0 || p.n_groups <= 0 || p.n_kv_blocks <= 0) return hipSuccess;
-    hipLaunchKernelGGL(bwd_hull_kernel, dim3(p.n_groups, p.B), dim3(64), 0, st, p);
-    hipError_t e = hipGetLastError();
+    const hipError_t e = launch1(bwd_hull_kernel, dim3(p.n_groups, p.B), dim3(64), st, p);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), 0, st, p);
-    return hipGetLastError();
+    return launch1(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), st, p);
 }
 
 hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.M * p.heads;
     if (rows == 0) return hipSuccess;
     const int grid = (int)std::min<int64_t>((rows + 15) / 16, 2048);
-    if (p.f16) hipLaunchKernelGGL(norm_bwd_kernel<true>, dim3(grid), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(norm_bwd_kernel<false>, dim3(grid), dim3(256), 0, st, p);
-    return hipGetLastError();
+    if (p.f16) return launch1(norm_bwd_kernel<true>, dim3(grid), dim3(256), st, p);
+    else return launch1(norm_bwd_kernel<false>, dim3(grid), dim3(256), st, p);
 }
 
 hipError_t launch_cast(const CastParams& p, hipStream_t st) {
@@ -352,13 +349,12 @@ hipError_t launch_cast(const CastParams& p, hipStream_t st) {
     if (rows == 0) return hipSuccess;
     const dim3 grid(blocks_for(rows));
     if (p.transposed) {
-        if (p.f16) hipLaunchKernelGGL(cast_t_kernel<true>, grid, dim3(256), 0, st, p);
-        else hipLaunchKernelGGL(cast_t_kernel<false>, grid, dim3(256), 0, st, p);
+        if (p.f16) return launch1(cast_t_kernel<true>, grid, dim3(256), st, p);
+        else return launch1(cast_t_kernel<false>, grid, dim3(256), st, p);
     } else {
-        if (p.f16) hipLaunchKernelGGL(cast_kernel<true>, grid, dim3(256), 0, st, p);
-        else hipLaunchKernelGGL(cast_kernel<false>, grid, dim3(256), 0, st, p);
+        if (p.f16) return launch1(cast_kernel<true>, grid, dim3(256), st, p);
+        else return launch1(cast_kernel<false>, grid, dim3(256), st, p);
     }
-    return hipGetLastError();
 }
 
 }  // namespace lvx

@@ -62,7 +62,11 @@ def _reject_unsupported(causal):
     if causal:
         # the reference applies the triangle to rank-local indices only
         # (lv_xattn/attn.py:229,237), which means nothing once blocks travel
-        raise ValueError("causal=True is not defined for cross-attention over travelling query blocks")
+        raise ValueError("causal=True is not defined for cross-attention over travelling query blocks: the "
+                         "reference applies the triangle to rank-local row and key indices only "
+                         "(lv_xattn/attn.py:229-237).  Its patched Mllama forward passes is_causal=True "
+                         "whenever there is no attention mask and more than one query (test_llama3.py:430); "
+                         "pass False there, cross-attention has no causal order")
 
 
 def _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, dev) -> Optional[torch.Tensor]:
@@ -80,7 +84,9 @@ def _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, de
         raise ValueError(f"bias_func must return [B|1, 1|Hq, {Lq}, {Lkv}], got {tuple(bias.shape)}")
     bias = bias.to(device=dev, dtype=torch.float32)
     pad = -Lkv % 4          # the kernels read a row in groups of 4 keys
-    if bias.stride(3) != 1 or bias.stride(2) < Lkv + pad:
+    # rows are read with 16-byte loads: aligned base, strides multiples of 4, rows readable up to Lkv + pad
+    strides_ok = all(bias.stride(i) % 4 == 0 or bias.shape[i] == 1 for i in range(3))
+    if bias.stride(3) != 1 or bias.stride(2) < Lkv + pad or not strides_ok or bias.data_ptr() % 16:
         padded = torch.zeros(*bias.shape[:3], Lkv + pad, dtype=torch.float32, device=dev)
         padded[..., :Lkv] = bias
         bias = padded[..., :Lkv]

@@ -18,7 +18,7 @@ from typing import Callable, Optional
 import torch
 
 from . import ops
-from .attn import Mask, _attn_backward, _attn_forward
+from .attn import Mask, _attn_backward, _attn_forward, _reject_unsupported
 from .async_communication import reset_global_memory_buffer
 
 
@@ -70,8 +70,17 @@ class KVProjection:
 def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = False,
                            rounds: Optional[int] = None, batched: bool = False,
                            weight_grads: bool = False, w_in_major: bool = True):
-    """apply(q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None, k_norm_weight=None,
-    k_norm_eps=1e-5, bias_func=None, *bias_args) -> o
+    """Two call shapes, told apart by their arguments.
+
+    apply(x, run_function, is_causal) -> o: the reference's (test_llama3.py:184-243, called at
+    :459 as attention(hidden_states, project, is_causal)).  q, k, v = run_function(x,
+    get_global_cross_attention_states()); saves (x, o, L) only; backward runs run_function
+    again and sends dq, dk, dv back through it (real gradients, where the reference returns
+    None).  Build run_function from `create_q_projection_class` / `create_kv_projection_class`
+    to keep every GEMM on this library's kernels.
+
+    apply(q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None, k_norm_weight=None,
+    k_norm_eps=1e-5, bias_func=None, *bias_args) -> o: q given, K/V recomputed:
 
     Forward: K, V = kv_proj(x_vis); o, L = attention; saves (q, x_vis, w_k, w_v,
     o, L) - K and V are dropped.  Backward: recomputes K, V by the same GEMMs,
@@ -86,7 +95,7 @@ def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = 
     if attention_mode != "lv_xattn":
         raise ValueError("only attention_mode='lv_xattn' exists on this path")
 
-    class _attention(torch.autograd.Function):
+    class _attention_by_tensors(torch.autograd.Function):
         @staticmethod
         def forward(ctx, q, x_vis, w_k, w_v, n_kv_heads, sm_scale, mask=None, k_norm_weight=None,
                     k_norm_eps=1e-5, bias_func=None, *bias_args):
@@ -125,7 +134,112 @@ def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = 
                 dwk, dwv = ops.dw_kv(x_vis, dk, dv, w_in_major)
             return (dq, dx, dwk, dwv, None, None, None, dwn, None, None) + (None,) * ctx.n_bias
 
+    class _attention_by_run_function(torch.autograd.Function):
+        # The reference's own call shape (test_llama3.py:184-243): apply(x, run_function, is_causal)
+        # with q, k, v = run_function(x, get_global_cross_attention_states()) and
+        # sm_scale = head_dim ** -0.5.  Only (x, o, L) are kept; backward runs run_function again -
+        # under autograd, on a detached x - and pushes dq, dk, dv back through it, so x gets its
+        # gradient and so does whatever else run_function's graph reaches (projection weights,
+        # norm weights, the visual states), where the reference returns none (:243).
+        @staticmethod
+        def forward(ctx, x, run_function, is_causal):
+            _reject_unsupported(is_causal)
+            q, k, v = run_function(x, get_global_cross_attention_states())
+            sm_scale = q.size(-1) ** -0.5
+            _, _, _, o, L = _attn_forward(q, k, v, is_causal, sm_scale, None, None, [], [], no_overlap,
+                                          rounds=rounds, batched=batched)
+            ctx.save_for_backward(x, o, L)
+            ctx.run_function, ctx.causal = run_function, is_causal
+            reset_global_memory_buffer(attention_mode)
+            return o
+
+        @staticmethod
+        def backward(ctx, do):
+            x, o, L = ctx.saved_tensors
+            x_ = x.detach().requires_grad_(x.requires_grad)
+            with torch.enable_grad():
+                q, k, v = ctx.run_function(x_, get_global_cross_attention_states())
+            sm_scale = q.size(-1) ** -0.5
+            dq, dk, dv = _attn_backward(do, q.detach(), k.detach(), v.detach(), o, L, ctx.causal, sm_scale, None,
+                                        "flash", None, [], [], no_overlap, rounds=rounds, batched=batched)
+            outs = [(t, g) for t, g in ((q, dq), (k, dk), (v, dv)) if t.requires_grad]
+            if outs:
+                torch.autograd.backward([t for t, _ in outs], [g for _, g in outs])
+            reset_global_memory_buffer(attention_mode)
+            return x_.grad, None, None
+
+    class _attention:
+        """`apply` takes either call shape: (x, run_function, is_causal) - the reference's - or
+        (q, x_vis, w_k, w_v, n_kv_heads, sm_scale, ...)."""
+        by_tensors, by_run_function = _attention_by_tensors, _attention_by_run_function
+
+        @staticmethod
+        def apply(*args):
+            if len(args) == 3 and callable(args[1]):
+                return _attention_by_run_function.apply(*args)
+            return _attention_by_tensors.apply(*args)
+
     return _attention
+
+
+_global_cross_attention_states = None
+
+
+def set_global_cross_attention_states(vision_features):
+    """The visual hidden states every cross-attention layer projects its K and V from
+    (test_llama3.py:69-79): set once per step, read by the run_function wrapper in both passes."""
+    global _global_cross_attention_states
+    _global_cross_attention_states = vision_features
+
+
+def get_global_cross_attention_states():
+    return _global_cross_attention_states
+
+
+def clear_global_cross_attention_states():
+    global _global_cross_attention_states
+    _global_cross_attention_states = None
+
+
+def create_kv_projection_class(w_in_major: bool = True, weight_grads: bool = True):
+    """apply(x_vis, w_k, w_v, n_kv_heads, k_norm_weight=None, eps=1e-5) -> k, v [B, Hkv, Lkv, D]
+
+    The visual side of the reference's `project` (test_llama3.py:395-398, 418) as one autograd
+    function over the fused GEMMs: K = k_norm(X_vis W_k), V = X_vis W_v.  Nothing but the inputs
+    is kept; backward re-runs the projection for the raw K and its r when there is a norm, goes
+    back through the norm, then dX_vis = dK W_k^T + dV W_v^T and (weight_grads) dW_k, dW_v and
+    the norm weight's gradient."""
+
+    class _kv_projection(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x_vis, w_k, w_v, n_kv_heads, k_norm_weight=None, eps=1e-5):
+            ctx.has_norm = k_norm_weight is not None
+            ctx.save_for_backward(x_vis, w_k, w_v, *([k_norm_weight] if ctx.has_norm else []))
+            ctx.n_kv_heads, ctx.eps = n_kv_heads, eps
+            return ops.kv_proj(x_vis, w_k, w_v, n_kv_heads, w_in_major, k_norm_weight=k_norm_weight, eps=eps)
+
+        @staticmethod
+        def backward(ctx, dk, dv):
+            x_vis, w_k, w_v, *rest = ctx.saved_tensors
+            dwn = None
+
+            def token_major(t):      # [B, H, L, D] gradients in [B, L, H, D] memory order, as the GEMMs read them
+                return t if t.transpose(1, 2).is_contiguous() else t.transpose(1, 2).contiguous().transpose(1, 2)
+
+            dk, dv = token_major(dk), token_major(dv)
+            if ctx.has_norm:
+                _, _, k_raw, k_rstd = ops.kv_proj(x_vis, w_k, w_v, ctx.n_kv_heads, w_in_major, k_norm_weight=rest[0],
+                                                  eps=ctx.eps, for_backward=True)
+                dk, dwn = ops.k_norm_bwd(dk, k_raw, k_rstd, rest[0], want_dw=weight_grads)
+                if dwn is not None:
+                    dwn = dwn.to(rest[0].dtype)
+            dx = ops.dx_vis(dk, dv, w_k, w_v, w_in_major)
+            dwk = dwv = None
+            if weight_grads:
+                dwk, dwv = ops.dw_kv(x_vis, dk, dv, w_in_major)
+            return dx, dwk, dwv, None, dwn, None
+
+    return _kv_projection
 
 
 def create_q_projection_class(w_in_major: bool = True, weight_grads: bool = True):

@@ -67,6 +67,8 @@ def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask],
             raise LvxError(f"bias must be an fp32 [B|1, Hq|1, {Lq}, {Lkv}] tensor with unit last stride on {q.device}")
         if bias.stride(2) < (Lkv + 3) // 4 * 4:
             raise LvxError("bias rows must be padded to a multiple of 4 floats (row stride >= Lkv rounded up to 4)")
+        if bias.data_ptr() % 16 or any(bias.stride(i) % 4 and bias.shape[i] > 1 for i in range(3)):
+            raise LvxError("bias must be 16-byte aligned with batch, head and row strides that are multiples of 4 floats")
         s.bias = bias.data_ptr()
         s.bias_stride_b = bias.stride(0) if bias.shape[0] > 1 else 0
         s.bias_stride_h = bias.stride(1) if bias.shape[1] > 1 else 0

@@ -80,6 +80,16 @@ def test_forward_rejects_bad_arguments_before_launch(lib):
     assert lib.lvx_fwd(None, None, None, None, None, None, 0, 0, 1, None, 0, None) == -1
 
 
+def test_dense_bias_must_be_aligned_for_16_byte_loads(lib):
+    ok = dict(bias=0x8000, bias_stride_b=64 * 256, bias_stride_h=0, bias_stride_r=256)
+    assert _fwd(lib, _shape(**ok), rc=0) == 0                       # accepted (no rows: nothing is launched)
+    assert _fwd(lib, _shape(**dict(ok, bias=0x8004))) == -2         # base not 16-byte aligned
+    assert _fwd(lib, _shape(**dict(ok, bias_stride_r=257))) == -2   # rows would start off a 16-byte boundary
+    assert _fwd(lib, _shape(**dict(ok, bias_stride_b=64 * 256 + 2))) == -2
+    assert _fwd(lib, _shape(**dict(ok, bias_stride_h=6))) == -2
+    assert _fwd(lib, _shape(**dict(ok, bias_stride_r=252))) == -3   # shorter than Lkv rounded up to 4
+
+
 def test_workspace_size(lib):
     s = _shape()
     assert lib.lvx_fwd_workspace_bytes(C.byref(s), 64, 1) == 0
@@ -109,6 +119,15 @@ def test_other_entry_points_reject_bad_arguments(lib):
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need - 1, None) == -7
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, None, 0, None) == -7
+    # row offsets of q and dO are formed in 32 bits: Lq * row stride must stay below 2^31
+    big = _shape(Lq=1 << 20, Lkv=128)
+    wide = _t(sb=1 << 40, sh=1 << 33, ss=2048)          # 2^20 rows x 2048 elements = 2^31
+    need_big = lib.lvx_bwd_workspace_bytes(C.byref(big), 64)
+    assert lib.lvx_bwd(C.byref(big), C.byref(wide), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
+                       C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need_big, None) == -8
+    assert lib.lvx_bwd(C.byref(big), C.byref(t), C.byref(t), C.byref(t), C.byref(wide), 0x2000, 0x2000, C.byref(t),
+                       C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need_big, None) == -8
+    assert b"not supported" in lib.lvx_strerror(-8)
     assert lib.lvx_cast_f32(0x1000, C.byref(t), 1, 8, 64, 64, 1, None) == -4
     assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, 1, None) == -3
     assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, 2, None) == -1

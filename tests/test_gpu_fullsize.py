@@ -1,9 +1,8 @@
 """GPU parity at the full sizes of the five benchmark configurations.
 
-cfg2, cfg3 and cfg4 are compared against the CPU oracle in full (tens of
-seconds of host time each); cfg1 against the oracle on two of its eight kv
-heads, plus size-independent properties (batched == per-round bit for bit,
-key splits within tolerance, rows of P sum to one)."""
+cfg1, cfg2, cfg3 and cfg4 are compared against the CPU oracle in full (tens of
+seconds of host time each), plus size-independent properties (batched ==
+per-round bit for bit, key splits within tolerance, rows of P sum to one)."""
 import pytest
 import torch
 
@@ -52,8 +51,8 @@ def test_cfg1_forward_full_size(lvx):
     _, _, _, o_a, l_a = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds)
     torch.cuda.synchronize()
     assert (o_r.float() - o_a.float()).abs().max() <= 2e-2 and (l_r - l_a).abs().max() <= 1e-3
-    # oracle on kv heads 0 and 5 (q heads 0-3 and 20-23), all rows, all keys
-    for hk in (0, 5):
+    # the oracle, one kv head (4 q heads) at a time: all rows, all keys
+    for hk in range(w.Hkv):
         hs = slice(4 * hk, 4 * hk + 4)
         o_ref, l_ref = orc.round_loop_forward(t["q"][:, hs], t["k"][:, hk:hk + 1], t["v"][:, hk:hk + 1],
                                               w.scale, w.rounds)
@@ -96,11 +95,26 @@ def test_cfg2_layer_full_size(lvx, batched):
 
 def test_cfg3_long_video_full_size(lvx):
     w = orc.make_inputs(orc.workload("cfg3"))
+    t = w.tensors
     ref = orc.layer_reference(w)
     o, dq, dx, _, _ = _layer_on_device(lvx, w, batched=True)
     check_o(o, ref["o"])
     check_grad(dq, ref["dq"], "dQ")
     check_grad(dx, ref["dx_vis"], "dX_vis")
+    del o, dq, dx
+    # one launch per round (16 rounds of 128 rows against 65536 keys), operators called as
+    # the round loops call them, with dK and dV checked directly
+    from lv_xattn import ops
+    q, do = _dev(t["q"]), _dev(t["do"])
+    k, v = ops.kv_proj(_dev(t["x_vis"]), _dev(t["w_k"]), _dev(t["w_v"]), w.Hkv)
+    _, _, _, o, L = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, batched=False)
+    dq, dk, dv = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash", rounds=w.rounds, batched=False)
+    torch.cuda.synchronize()
+    check_o(o, ref["o"])
+    check_lse(L, ref["lse"])
+    check_grad(dq, ref["dq"], "dQ (per round)")
+    check_grad(dk, ref["dk"], "dK (per round)")
+    check_grad(dv, ref["dv"], "dV (per round)")
 
 
 @pytest.mark.parametrize("batched", [True, False])
@@ -122,6 +136,43 @@ def test_cfg4_masked_ragged_full_size(lvx, batched):
     dead = torch.isinf(ref["lse"])
     assert dead.any() and (o.float().cpu()[dead] == 0).all() and (dq.float().cpu()[dead] == 0).all()
     assert (dk.float().cpu()[1, :, w.kv_len[1]:] == 0).all()
+
+
+def test_cfg4_full_size_through_the_dense_bias_variant(lvx):
+    """cfg4's interval mask written as the reference would pass it: a dense additive bias
+    [B, 1, Lq, Lkv] of 0 / -inf through bias_func (lv_xattn/attn.py:386-389).  Same answer as the
+    interval-mask kernels and as the oracle."""
+    w = orc.make_inputs(orc.workload("cfg4"))
+    t = w.tensors
+    ref = orc.layer_reference(w)
+    q, k, v, do = (_dev(t[n]) for n in ("q", "k", "v", "do"))
+    keys = torch.arange(w.Lkv).view(1, 1, 1, -1)
+    kv_len = torch.tensor(w.kv_len).view(-1, 1, 1, 1)
+    seen = (keys >= t["kv_start"].view(w.B, 1, w.Lq, 1)) & (keys < t["kv_end"].view(w.B, 1, w.Lq, 1)) & (keys < kv_len)
+    bias = torch.zeros(w.B, 1, w.Lq, w.Lkv).masked_fill_(~seen, float("-inf"))
+    bias_d = _dev(bias)
+    del bias, seen
+    _, _, _, o, L = lvx._attn_forward(q, k, v, False, w.scale, None, lambda b_: b_, [bias_d], [], rounds=w.rounds,
+                                      batched=True)
+    dq, dk, dv = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash", lambda b_: b_, [bias_d], [],
+                                    rounds=w.rounds, batched=True)
+    mask = _mask_of(w, lvx)
+    _, _, _, o_m, L_m = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, mask=mask, batched=True)
+    dq_m, dk_m, dv_m = lvx._attn_backward(do, q, k, v, o_m, L_m, False, w.scale, None, "flash", rounds=w.rounds,
+                                          mask=mask, batched=True)
+    torch.cuda.synchronize()
+    check_o(o, ref["o"])
+    check_lse(L, ref["lse"])
+    check_grad(dq, ref["dq"], "dQ")
+    check_grad(dk, ref["dk"], "dK")
+    check_grad(dv, ref["dv"], "dV")
+    # the two mask forms agree far more closely than either has to agree with the oracle
+    assert (o.float() - o_m.float()).abs().max() <= 4e-3
+    fin = ~torch.isinf(L_m)
+    assert torch.equal(torch.isinf(L), torch.isinf(L_m)) and (L[fin] - L_m[fin]).abs().max() <= 1e-4
+    for a, b_, what in ((dq, dq_m, "dQ"), (dk, dk_m, "dK"), (dv, dv_m, "dV")):
+        scale = b_.float().abs().max()
+        assert (a.float() - b_.float()).abs().max() <= 4e-3 * scale, what
 
 
 @pytest.mark.parametrize("name", ["cfg2", "cfg4"])

@@ -136,7 +136,96 @@ def test_q_projection_with_q_norm_autograd(lvx, w_in_major, dtype):
     check_grad(wnd.grad, dwn_ref, "dw_norm")
 
 
+def test_reference_call_shape_of_the_recompute_wrapper(lvx):
+    """attention(hidden_states, project, is_causal) exactly as the reference's patched forward calls
+    it (test_llama3.py:184-243, 459): q, k, v come from run_function(x, global visual states) in
+    both passes, only (x, o, L) are kept, and - unlike the reference (:243) - every input of the
+    projection gets its gradient.  Checked against the oracle's layer (projection with q_norm /
+    k_norm, attention, backward through all of it)."""
+    g = torch.Generator().manual_seed(21)
+    B, Lq, Lkv, Dm, Hq, Hkv, D = 2, 96, 301, 256, 8, 2, 128
+    dt = torch.bfloat16
+    x = (torch.randn(B, Lq, Dm, generator=g) * 0.5).to(dt)
+    vis = (torch.randn(B, Lkv, Dm, generator=g) * 0.5).to(dt)
+    wq = (torch.randn(Dm, Hq * D, generator=g) * 0.08).to(dt)
+    wk = (torch.randn(Dm, Hkv * D, generator=g) * 0.08).to(dt)
+    wv = (torch.randn(Dm, Hkv * D, generator=g) * 0.08).to(dt)
+    wqn = (1.0 + 0.2 * torch.randn(D, generator=g)).to(dt)
+    wkn = (1.0 + 0.2 * torch.randn(D, generator=g)).to(dt)
+    do = torch.randn(B, Hq, Lq, D, generator=g).to(dt)
+    scale = D ** -0.5
+    # oracle: projections (rounded to bf16 where the device stores them), norms, attention, all the way back
+    q_raw, _ = orc.kv_project(x, wq, wq, Hq)
+    q_raw = q_raw.to(dt)
+    q_ref = orc.k_rms_norm(q_raw, wqn, 1e-5).to(dt)
+    k_raw, v_ref = orc.kv_project(vis, wk, wv, Hkv)
+    k_raw, v_ref = k_raw.to(dt), v_ref.to(dt)
+    k_ref = orc.k_rms_norm(k_raw, wkn, 1e-5).to(dt)
+    o_ref, l_ref = orc.round_loop_forward(q_ref, k_ref, v_ref, scale, 1)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q_ref, k_ref, v_ref, o_ref, l_ref, scale)
+    dq_raw_ref, dwqn_ref = orc.k_rms_norm_backward(dq_ref.to(dt), q_raw, wqn, 1e-5)
+    dk_raw_ref, dwkn_ref = orc.k_rms_norm_backward(dk_ref.to(dt), k_raw, wkn, 1e-5)
+    dx_ref = orc.dx_vis(dq_raw_ref.to(dt), torch.zeros_like(dq_raw_ref), wq, wq)
+    dvis_ref = orc.dx_vis(dk_raw_ref.to(dt), dv_ref.to(dt), wk, wv)
+    dwq_ref, _ = orc.dw_kv(x, dq_raw_ref.to(dt), torch.zeros_like(dq_raw_ref))
+    dwk_ref, dwv_ref = orc.dw_kv(vis, dk_raw_ref.to(dt), dv_ref.to(dt))
+
+    xd, visd = _dev(x).requires_grad_(), _dev(vis).requires_grad_()
+    wqd, wkd, wvd = (_dev(t).requires_grad_() for t in (wq, wk, wv))
+    wqnd, wknd = _dev(wqn).requires_grad_(), _dev(wkn).requires_grad_()
+    q_proj, kv_proj = lvx.create_q_projection_class().apply, lvx.create_kv_projection_class().apply
+    calls = []
+
+    def project(hidden_states, cross_attention_states):      # the reference's closure, on this library's GEMMs
+        calls.append(torch.is_grad_enabled())
+        query_states = q_proj(hidden_states, wqd, Hq, wqnd, 1e-5)
+        key_states, value_states = kv_proj(cross_attention_states, wkd, wvd, Hkv, wknd, 1e-5)
+        return query_states, key_states, value_states
+
+    attention = lvx.create_attention_class("lv_xattn", no_overlap=False).apply
+    lvx.set_global_cross_attention_states(visd)
+    try:
+        o = attention(xd, project, False)
+        assert len(o.grad_fn.saved_tensors) == 3        # x, o, L: neither Q nor K nor V is kept
+        o.backward(_dev(do))
+        torch.cuda.synchronize()
+    finally:
+        lvx.clear_global_cross_attention_states()
+    assert calls == [False, True]                        # forward without a graph, backward's recompute with one
+    check_o(o.detach(), o_ref)
+    check_grad(xd.grad, dx_ref, "dX")
+    check_grad(visd.grad, dvis_ref, "dX_vis")
+    check_grad(wqd.grad, dwq_ref, "dW_q")
+    check_grad(wkd.grad, dwk_ref, "dW_k")
+    check_grad(wvd.grad, dwv_ref, "dW_v")
+    check_grad(wqnd.grad, dwqn_ref, "dw_q_norm")
+    check_grad(wknd.grad, dwkn_ref, "dw_k_norm")
+    with pytest.raises(ValueError, match=r"test_llama3\.py:430"):
+        attention(xd, project, True)
+
+
 # ------------------------------------------------------------------ row-wise kernels
+def test_merge_ignores_an_accumulator_that_holds_nothing_yet(lvx):
+    """(garbage, L = -inf) is the identity of the merge: a travelling accumulator may start as
+    uninitialised memory with L = -inf, whatever bits its O holds."""
+    from lv_xattn import ops
+    g = torch.Generator().manual_seed(9)
+    B, H, L, D = 1, 2, 40, 128
+    ob = torch.randn(B, H, L, D, generator=g).bfloat16()
+    lb = torch.randn(B, H, L, generator=g) + 5
+    lb[0, 1, 7] = float("-inf")                         # a part that saw no key either
+    o_acc = torch.full((B, H, L, D), float("nan")).bfloat16()
+    o_acc[0, 0, 1] = float("inf")
+    l_acc = torch.full((B * H, L), float("-inf"))
+    o_d, l_d = _dev(o_acc), _dev(l_acc)
+    ops.merge(o_d, l_d, _dev(ob), _dev(lb).reshape(B * H, L).contiguous())
+    torch.cuda.synchronize()
+    want = ob.clone()
+    want[0, 1, 7] = 0
+    assert torch.equal(o_d.cpu(), want)
+    assert torch.equal(l_d.cpu(), lb.reshape(B * H, L))
+
+
 def test_merge_against_oracle(lvx):
     from lv_xattn import ops
     g = torch.Generator().manual_seed(7)

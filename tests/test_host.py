@@ -58,6 +58,15 @@ def test_causal_and_malformed_bias_are_rejected_explicitly():
         lv_xattn._attn_forward(q, k, k, False, 0.1, None, local_bias_args=[torch.zeros(1)])
     with pytest.raises(ValueError, match="causal"):
         lv_xattn._attn_backward(q, q, k, k, q, torch.zeros(4, 8), True, 0.1, None, "flash")
+    # the reference's patched Mllama forward passes is_causal=True when there is no mask and
+    # more than one query (test_llama3.py:430): the refusal says where that comes from, in the
+    # round loops and in both autograd wrappers
+    with pytest.raises(ValueError, match=r"test_llama3\.py:430"):
+        lv_xattn._attn_forward(q, k, k, True, 0.1, None)
+    with pytest.raises(ValueError, match=r"test_llama3\.py:430"):
+        lv_xattn.create_attention_class_save_qkv("lv_xattn").apply(q, k, k, True, 0.1)
+    with pytest.raises(ValueError, match=r"test_llama3\.py:430"):
+        lv_xattn.create_attention_class("lv_xattn").apply(q, lambda x, vis: (q, k, k), True)
 
 
 def test_shape_and_dtype_checks_raise_before_any_device_call():
