@@ -17,6 +17,9 @@ import torch
 _ROUNDS = 1
 _INITIALISED = False
 _WORKSPACES: Dict[Tuple, torch.Tensor] = {}
+# Largest dS^T workspace one backward call may use; larger row windows are cut into chunks
+# (see set_backward_workspace_cap)
+_BWD_WS_CAP = int(float(os.environ.get("LVX_BWD_WS_CAP_GB", "12")) * (1 << 30))
 
 
 class _RoundGroup:
@@ -76,11 +79,39 @@ def reset_global_memory_buffer(*_ignored) -> None:
     _WORKSPACES.clear()
 
 
+def set_backward_workspace_cap(nbytes: int) -> None:
+    """The backward keeps scale*dS for a whole row window in a workspace of
+    2 bytes x B x Hq x Lkv (rounded up to 128) x rows: 1.7 GB at B1 Hq32 Lq4096 Lkv6404, 13.7 GB at
+    B8.  A window whose workspace would exceed `nbytes` is run as several calls over row chunks
+    (dK / dV accumulate in fp32 across them), which costs a few per cent per extra call.
+    Default 12 GiB, or LVX_BWD_WS_CAP_GB."""
+    global _BWD_WS_CAP
+    if nbytes < (64 << 20):
+        raise ValueError("the cap must leave room for at least one chunk of rows (64 MiB or more)")
+    _BWD_WS_CAP = int(nbytes)
+
+
+def backward_workspace_cap() -> int:
+    return _BWD_WS_CAP
+
+
 def workspace(tag: str, shape, dtype, device) -> torch.Tensor:
-    """A cached scratch tensor; contents are undefined on return."""
-    key = (tag, tuple(shape), dtype, str(device))
-    t = _WORKSPACES.get(key)
-    if t is None:
-        t = torch.empty(*shape, dtype=dtype, device=device)
-        _WORKSPACES[key] = t
-    return t
+    """A cached scratch tensor; contents are undefined on return.  One buffer per (tag, device,
+    stream), grown to the largest size asked for so far: changing shapes (variable-length
+    batches) reuse it instead of adding a buffer per shape, and two streams never share one."""
+    dev = torch.device(device)
+    if dev.type == "cuda" and dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    stream = torch.cuda.current_stream(dev).cuda_stream if dev.type == "cuda" else 0
+    key = (tag, str(dev), stream)
+    numel = 1
+    for n in shape:
+        numel *= int(n)
+    nbytes = numel * torch.empty((), dtype=dtype).element_size()
+    buf = _WORKSPACES.get(key)
+    if buf is None or buf.numel() < nbytes:
+        _WORKSPACES.pop(key, None)
+        buf = None                       # the old buffer is released before the larger one is asked for
+        buf = torch.empty((nbytes + 255) // 256 * 256, dtype=torch.uint8, device=dev)
+        _WORKSPACES[key] = buf
+    return buf[:nbytes].view(dtype).view(*shape)

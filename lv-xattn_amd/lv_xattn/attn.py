@@ -20,7 +20,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 from . import ops
-from .async_communication import get_sequence_parallel_size, workspace
+from .async_communication import backward_workspace_cap, get_sequence_parallel_size, workspace
 from .ops import Mask
 
 __all__ = ["_attn_forward", "_attn_backward", "q_block_bounds", "Mask"]
@@ -161,6 +161,22 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     return q, k, v, o, L
 
 
+def _cap_windows(windows, nbytes_of_rows, cap):
+    """Cuts every row window whose backward workspace would exceed `cap` bytes into chunks of
+    whole 256-row groups that fit (the workspace grows linearly with the rows of a call)."""
+    out = []
+    for r0, r1 in windows:
+        rows = r1 - r0
+        if rows <= 256 or nbytes_of_rows(rows) <= cap:
+            out.append((r0, r1))
+            continue
+        chunk = rows
+        while chunk > 256 and nbytes_of_rows(chunk) > cap:
+            chunk = max(256, (chunk // 2 + 255) // 256 * 256)
+        out.extend((a, min(a + chunk, r1)) for a in range(r0, r1, chunk))
+    return out
+
+
 def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engine,
                    bias_func=None, local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
                    rounds: Optional[int] = None, mask: Optional[Mask] = None, batched: bool = False):
@@ -190,6 +206,7 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     dv = torch.empty(B, Lkv, Hkv, D, dtype=q_.dtype, device=dev).transpose(1, 2)
 
     windows = [(0, Lq)] if batched else [w for w in q_block_bounds(Lq, P) if w[1] > w[0]]
+    windows = _cap_windows(windows, lambda rows: ops.bwd_workspace_bytes(q_, k_, rows, mask), backward_workspace_cap())
     ws = workspace("bwd_ds", (ops.bwd_workspace_bytes(q_, k_, max(r1 - r0 for r0, r1 in windows), mask),),
                    torch.uint8, dev)
     if len(windows) == 1:

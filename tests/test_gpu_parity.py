@@ -377,6 +377,37 @@ def test_backward_cfg1s(lvx, batched):
     check_grad(dv, ref["dv"], "dV")
 
 
+def test_backward_in_row_chunks_under_a_small_workspace_cap(lvx):
+    """A window whose dS^T workspace would exceed the cap runs as several calls over row chunks
+    (fp32 dK / dV across them): same gradients as the single call."""
+    from lv_xattn import async_communication as ac
+    w = orc.workload("cfg1s")
+    w.Lq, w.rounds = 1024, 1
+    w = orc.make_inputs(w)
+    t = w.tensors
+    ref = orc.layer_reference(w)
+    q, k, v, do = (_dev(t[n]) for n in ("q", "k", "v", "do"))
+    _, _, _, o, L = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=1, batched=True)
+    one = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash", rounds=1, batched=True)
+    old = ac.backward_workspace_cap()
+    seen = []
+    real = ops_bwd = None
+    from lv_xattn import ops
+    real = ops.bwd
+    try:
+        ac._BWD_WS_CAP = ops.bwd_workspace_bytes(q, k, 300)      # forces chunks of 256 rows
+        ops.bwd = lambda *a, **kw: (seen.append((a[10], a[11])), real(*a, **kw))[1]
+        cut = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash", rounds=1, batched=True)
+    finally:
+        ops.bwd = real
+        ac._BWD_WS_CAP = old
+    torch.cuda.synchronize()
+    assert seen == [(0, 256), (256, 256), (512, 256), (768, 256)]
+    for g, g1, r, what in zip(cut, one, (ref["dq"], ref["dk"], ref["dv"]), ("dQ", "dK", "dV")):
+        check_grad(g, r, what)
+        assert (g.float() - g1.float()).abs().max() <= 2e-2 * r.abs().max()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("batched", [False, True])
 def test_cfg0_shape_head_dim_64_runs_zero_padded(lvx, batched, dtype):

@@ -40,11 +40,36 @@ def test_round_group_shim(monkeypatch):
 
 
 def test_workspace_cache_and_reset():
-    a = ac.workspace("t", (4, 4), torch.float32, "cpu")
-    assert ac.workspace("t", (4, 4), torch.float32, "cpu") is a
     lv_xattn.reset_global_memory_buffer()
-    assert ac.workspace("t", (4, 4), torch.float32, "cpu") is not a
+    a = ac.workspace("t", (4, 4), torch.float32, "cpu")
+    assert tuple(a.shape) == (4, 4) and a.dtype == torch.float32
+    # one buffer per tag: the same memory for the same or a smaller request, whatever the shape ...
+    assert ac.workspace("t", (4, 4), torch.float32, "cpu").data_ptr() == a.data_ptr()
+    assert ac.workspace("t", (2, 3), torch.bfloat16, "cpu").data_ptr() == a.data_ptr()
+    # ... grown (not multiplied) by a larger one
+    b = ac.workspace("t", (64, 64), torch.float32, "cpu")
+    assert tuple(b.shape) == (64, 64) and len(ac._WORKSPACES) == 1
+    assert ac.workspace("t", (4, 4), torch.float32, "cpu").data_ptr() == b.data_ptr()
+    assert ac.workspace("u", (4,), torch.float32, "cpu").data_ptr() != b.data_ptr() and len(ac._WORKSPACES) == 2
+    lv_xattn.reset_global_memory_buffer()
+    assert len(ac._WORKSPACES) == 0
     lv_xattn.reset_global_memory_buffer("lv_xattn")      # the reference passes the mode
+
+
+def test_backward_row_windows_are_cut_to_the_workspace_cap():
+    per_row = 2 * 8 * 32 * 6528                 # bytes of dS^T per text row at B8 Hq32 Lkv6404 (6528 = 51 x 128)
+    nbytes = lambda rows: per_row * ((rows + 31) // 32 * 32) + (1 << 20)
+    # under the cap: untouched
+    assert attn._cap_windows([(0, 4096)], nbytes, 14 << 30) == [(0, 4096)]
+    # over it: chunks of whole 256-row groups that fit, covering the window exactly
+    cut = attn._cap_windows([(0, 4096)], nbytes, 4 << 30)
+    assert cut[0][0] == 0 and cut[-1][1] == 4096 and all(a[1] == b[0] for a, b in zip(cut, cut[1:]))
+    assert all(nbytes(r1 - r0) <= 4 << 30 and (r1 - r0) % 256 == 0 for r0, r1 in cut[:-1]) and len(cut) == 4
+    # per-round windows that already fit stay as they are; a 256-row window is never cut
+    assert attn._cap_windows([(0, 188), (188, 376)], nbytes, 1 << 30) == [(0, 188), (188, 376)]
+    assert attn._cap_windows([(0, 256)], nbytes, 1 << 20) == [(0, 256)]
+    with pytest.raises(ValueError):
+        ac.set_backward_workspace_cap(1 << 20)
 
 
 def test_causal_and_malformed_bias_are_rejected_explicitly():
