@@ -25,6 +25,7 @@ for p in (ROOT, os.path.join(ROOT, "lv-xattn_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+ROUND_STREAMS = 4            # streams the one-launch-per-round mode may spread its rounds over
 
 
 def bwd_traffic_bytes(name):
@@ -51,12 +52,12 @@ def flops(w, n_pairs):
 class Layer:
     """Device-side state of one benchmark layer and its step function."""
 
-    def __init__(self, w, mode, dev):
+    def __init__(self, w, mode, dev, streams=1):
         import torch
         import lv_xattn
         from lv_xattn import ops
         self.torch, self.ops, self.lvx = torch, ops, lv_xattn
-        self.w, self.mode = w, mode
+        self.w, self.mode, self.streams = w, mode, streams
         t = w.tensors
         self.q = t["q"].to(dev)
         self.do = t["do"].to(dev)
@@ -84,12 +85,13 @@ class Layer:
         # the travelling accumulator arrives as the identity (0, -inf) and every
         # block's partial is folded into it by the merge kernel
         _, _, _, o, L = self.lvx._attn_forward(self.q, k, v, False, self.w.scale, None, rounds=self.w.rounds,
-                                               mask=self.mask, acc_in=(self.o_in, self.l_in), batched=self.batched)
+                                               mask=self.mask, acc_in=(self.o_in, self.l_in), batched=self.batched,
+                                               streams=self.streams)
         return o, L
 
     def backward(self, k, v, o, L):
         dq, dk, dv = self.lvx._attn_backward(self.do, self.q, k, v, o, L, False, self.w.scale, None, "flash",
-                                             rounds=self.w.rounds, mask=self.mask, batched=self.batched)
+                                             rounds=self.w.rounds, mask=self.mask, batched=self.batched, streams=self.streams)
         dx = self.ops.dx_vis(dk, dv, self.wk, self.wv) if self.has_proj else None
         return dq, dk, dv, dx
 
@@ -215,6 +217,12 @@ def run_only(layer, which, n, torch):
         dk = torch.empty(B, Lkv, Hkv, D, dtype=w.dtype, device=dev).transpose(1, 2)
         dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
         fn = lambda: ops.bwd(layer.q, k, v, layer.do, L, delta, dq, dk, dv, w.scale, mask=layer.mask, workspace=bws)
+    elif which == "merge":
+        o2, l2 = o.clone(), L.clone()
+        fn = lambda: ops.merge(o2, l2, o, L)
+    elif which == "preprocess":
+        delta = torch.empty_like(L)
+        fn = lambda: ops.bwd_preprocess(o, layer.do, delta)
     elif which == "kv_proj":
         fn = layer.project
     else:
@@ -367,7 +375,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--no-others", action="store_true", help="skip the sub-records of cfg1, cfg3 and cfg4")
-    ap.add_argument("--only", choices=["fwd", "bwd", "kv_proj", "dx_vis", "copy"],
+    ap.add_argument("--only", choices=["fwd", "bwd", "kv_proj", "dx_vis", "merge", "preprocess", "copy"],
                     help="launch just this operator --steps times (for rocprofv3 counter runs); "
                          "'copy' is a 1 GiB device copy that calibrates FETCH_SIZE / WRITE_SIZE")
     a = ap.parse_args()
@@ -429,6 +437,12 @@ def main():
         ms2 = time_gpu(other.step, max(3, a.steps // 2), 2, torch)
         out["config"]["other_mode"] = {"mode": other.mode, "ms_per_step": round(ms2, 4),
                                        "tflops": round(step_flops / ms2 / 1e9, 2)}
+        if other.mode == "rounds":
+            # the rounds of a step touch disjoint rows: on one GPU they may overlap
+            over = Layer(w, "rounds", dev, streams=ROUND_STREAMS)
+            ms3 = time_gpu(over.step, max(3, a.steps // 2), 2, torch)
+            out["config"]["other_mode"]["overlapped"] = {
+                "streams": ROUND_STREAMS, "ms_per_step": round(ms3, 4), "tflops": round(step_flops / ms3 / 1e9, 2)}
     if not a.no_others and w.name == "cfg2" and a.dtype == "bf16":
         # the other GPU configurations under the same clock (the headline stays cfg2)
         del layer

@@ -264,14 +264,21 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
 // whole round.  Splitting the steps of every token block over `S` work-groups
 // (which then add their dK/dV with atomics) evens that out; S is chosen to
 // minimise ceil(blocks * S / CUs) / S with ranges of at least 32 steps.
+// CUs of the device that is current (the one the caller's stream belongs to), asked for once per device
+static int cu_count() {
+    static int cached[MAX_DEVICES];          // 0: not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return n;
+}
+
 static int choose_q_splits(int blocks, int steps) {
-    static const int n_cu = [] {      // initialised once, by whichever thread comes first
-        int dev = 0, n = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n = prop.multiProcessorCount;
-        return n > 0 ? n : 256;
-    }();
+    const int n_cu = cu_count();
     int best = 1;
     double best_cost = (double)((blocks + n_cu - 1) / n_cu);
     for (int S = 2; S <= 8; ++S) {

@@ -96,29 +96,105 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     if (chunk == 0) p.l_acc[(int64_t)bh * p.l_acc_bh + row] = den > 0.f ? ms + __logf(den) : -INFINITY;
 }
 
+// The same for one part folded into the accumulator (what lvx_merge does every round), two rows
+// per thread: every load of both rows is issued before the first use, so a thread keeps
+// 64 + 8 bytes in flight.  780 bytes per (row, head).
+template <bool F16>
+__global__ __launch_bounds__(256) void merge_pair_kernel(const MergeParams p) {
+    using E = Elt<F16>;
+    const int nrows = p.row_end - p.row_begin;
+    const int64_t total = (int64_t)p.B * p.Hq * nrows;
+    const int64_t half = (total + 1) / 2;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int chunk = (int)(idx & 15);
+    const int64_t r0 = idx >> 4;
+    if (r0 >= half) return;
+    int64_t rr[2] = {r0, r0 + half};
+    const bool ok1 = rr[1] < total;
+    if (!ok1) rr[1] = r0;
+    uint16_t* oa[2];
+    const uint16_t* op[2];
+    float* la_p[2];
+    float la[2], lb[2];
+    u32x4 ua[2], ub[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int row = p.row_begin + (int)(rr[k] % nrows);
+        const int bh = (int)(rr[k] / nrows);
+        const int b = bh / p.Hq, h = bh % p.Hq;
+        oa[k] = p.o_acc + b * p.oa.b + h * p.oa.h + (int64_t)row * p.oa.s + chunk * 8;
+        op[k] = p.o_part + b * p.op.b + h * p.op.h + (int64_t)row * p.op.s + chunk * 8;
+        la_p[k] = p.l_acc + (int64_t)bh * p.l_acc_bh + row;
+        la[k] = *la_p[k];
+        lb[k] = p.l_part[(int64_t)bh * p.l_part_bh + row];
+        ua[k] = *reinterpret_cast<const u32x4*>(oa[k]);
+        ub[k] = *reinterpret_cast<const u32x4*>(op[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        if (k == 1 && !ok1) break;
+        const float m = fmaxf(la[k], lb[k]);
+        const float ms = (m == -INFINITY) ? 0.f : m;
+        const float wa = __expf(la[k] - ms), wb = __expf(lb[k] - ms);
+        const float den = wa + wb;
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        // a side with weight 0 may hold anything (it saw no key, or nothing was folded in yet)
+        const float ca = wa * inv, cb = wb * inv;
+        float fa[8], fb[8];
+        unpack8<E>(ua[k], fa);
+        unpack8<E>(ub[k], fb);
+        u32x4 u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float x0 = (ca > 0.f ? fa[2 * j] * ca : 0.f) + (cb > 0.f ? fb[2 * j] * cb : 0.f);
+            const float x1 = (ca > 0.f ? fa[2 * j + 1] * ca : 0.f) + (cb > 0.f ? fb[2 * j + 1] * cb : 0.f);
+            u[j] = E::pack(x0, x1);
+        }
+        *reinterpret_cast<u32x4*>(oa[k]) = u;
+        if (chunk == 0) *la_p[k] = den > 0.f ? ms + __logf(den) : -INFINITY;
+    }
+}
+
+// delta = rowsum(O * dO): 16 lanes x 16 bytes per row and tensor, two rows per thread with all
+// four loads issued before the first use.  516 bytes per (row, head).
 template <bool F16>
 __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
     using E = Elt<F16>;
     const int nrows = p.row_end - p.row_begin;
+    const int64_t total = (int64_t)p.B * p.Hq * nrows;
+    const int64_t half = (total + 1) / 2;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int chunk = (int)(idx & 15);
-    const int64_t r = idx >> 4;
-    const bool ok = r < (int64_t)p.B * p.Hq * nrows;   // whole 16-lane groups share `ok`
-    const int64_t rr = ok ? r : 0;
-    const int row = p.row_begin + (int)(rr % nrows);
-    const int bh = (int)(rr / nrows);
-    const int b = bh / p.Hq, h = bh % p.Hq;
-    float fo[8], fd[8];
-    unpack8<E>(ldg16(p.o + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s + chunk * 8, ok), fo);
-    unpack8<E>(ldg16(p.dout + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8, ok), fd);
-    float s = 0.f;
+    const int64_t r0 = idx >> 4;
+    const bool ok0 = r0 < half;                         // whole 16-lane groups share the flags
+    const bool ok1 = ok0 && r0 + half < total;
+    const int64_t rr[2] = {ok0 ? r0 : 0, ok1 ? r0 + half : 0};
+    u32x4 uo[2], ud[2];
+    float* out[2];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
-    s += __shfl_xor(s, 8);
-    s += __shfl_xor(s, 4);
-    s += __shfl_xor(s, 2);
-    s += __shfl_xor(s, 1);
-    if (ok && chunk == 0) p.delta[(int64_t)bh * p.Lq + row] = s;
+    for (int k = 0; k < 2; ++k) {
+        const int row = p.row_begin + (int)(rr[k] % nrows);
+        const int bh = (int)(rr[k] / nrows);
+        const int b = bh / p.Hq, h = bh % p.Hq;
+        const bool ok = k ? ok1 : ok0;
+        uo[k] = ldg16(p.o + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s + chunk * 8, ok);
+        ud[k] = ldg16(p.dout + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8, ok);
+        out[k] = p.delta + (int64_t)bh * p.Lq + row;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        float fo[8], fd[8];
+        unpack8<E>(uo[k], fo);
+        unpack8<E>(ud[k], fd);
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
+        s += __shfl_xor(s, 8);
+        s += __shfl_xor(s, 4);
+        s += __shfl_xor(s, 2);
+        s += __shfl_xor(s, 1);
+        if ((k ? ok1 : ok0) && chunk == 0) *out[k] = s;
+    }
 }
 
 // LSE and delta of the window, re-expressed once for the backward kernel: the
@@ -308,6 +384,11 @@ inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
+    if (p.nparts == 1 && p.use_acc) {
+        const dim3 grid(blocks_for((rows + 1) / 2));
+        if (p.f16) return launch1(merge_pair_kernel<true>, grid, dim3(256), st, p);
+        return launch1(merge_pair_kernel<false>, grid, dim3(256), st, p);
+    }
     if (p.f16) return launch1(merge_kernel<true>, dim3(blocks_for(rows)), dim3(256), st, p);
     else return launch1(merge_kernel<false>, dim3(blocks_for(rows)), dim3(256), st, p);
 }
@@ -315,8 +396,8 @@ hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
 hipError_t launch_preprocess(const PreParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    if (p.f16) return launch1(preprocess_kernel<true>, dim3(blocks_for(rows)), dim3(256), st, p);
-    else return launch1(preprocess_kernel<false>, dim3(blocks_for(rows)), dim3(256), st, p);
+    if (p.f16) return launch1(preprocess_kernel<true>, dim3(blocks_for((rows + 1) / 2)), dim3(256), st, p);
+    else return launch1(preprocess_kernel<false>, dim3(blocks_for((rows + 1) / 2)), dim3(256), st, p);
 }
 
 hipError_t launch_bwd_meta(const MetaParams& p0, hipStream_t st) {

@@ -111,7 +111,7 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
                   local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
                   rounds: Optional[int] = None, mask: Optional[Mask] = None,
                   acc_in: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                  kv_splits: Optional[int] = None, batched: bool = False):
+                  kv_splits: Optional[int] = None, batched: bool = False, streams: int = 1):
     """Returns (q, k, v, o, L) like the reference (attn.py:435): o [B,Hq,Lq,D]
     bf16, L [B*Hq, Lq] fp32 natural-log LSE of sm_scale * q k^T.
 
@@ -123,7 +123,9 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     L_in fp32 [B*Hq,Lq]) for every block, `kv_splits` (key ranges per round
     computed by separate work-groups; default: enough to give every CU two
     work-groups, see auto_kv_splits), `batched` (one launch over all P blocks
-    instead of one per round)."""
+    instead of one per round), `streams` (the rounds of one call touch disjoint rows, so on one
+    GPU they may overlap: round r is queued on stream r % streams, the current stream and
+    streams - 1 others of the same priority, joined before the call returns)."""
     _reject_unsupported(causal)
     D_in = q.shape[-1]
     q_, k_, v_ = (_usable(_pad_head_dim(t)) for t in (q, k, v))
@@ -152,13 +154,53 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     # the partial goes straight into (o, L); an incoming accumulator is then folded into it
     # (the merge is symmetric, so which side is "the accumulator" does not matter, and neither
     # a copy of acc_in nor a buffer for the partial is needed)
-    for r0, r1 in windows:
+    def one_round(r0, r1, ws):
         ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
         if acc_in is not None:
             ops.merge(o, L, acc_o, acc_l, r0, r1 - r0)
+
+    if streams > 1 and len(windows) > 1:
+        with _RoundStreams(dev, min(streams, len(windows))) as rs:
+            for i, (r0, r1) in enumerate(windows):
+                with rs.stream(i):
+                    ws_i = workspace("fwd_split", (nbytes,), torch.uint8, dev) if kv_splits > 1 else None
+                    one_round(r0, r1, ws_i)
+    else:
+        for r0, r1 in windows:
+            one_round(r0, r1, ws)
     if D_in != D:
         o = o[..., :D_in].contiguous()
     return q, k, v, o, L
+
+
+class _RoundStreams:
+    """The current stream plus n - 1 side streams of the same (default) priority for the rounds
+    of one call.  The side streams start behind everything queued on the current stream so far;
+    on exit the current stream waits for all of them, so nothing that follows the call can see
+    a half-finished round and every tensor the rounds touched may be released as usual."""
+    _side = {}
+
+    def __init__(self, device, n):
+        self.dev, self.n = torch.device(device), n
+
+    def __enter__(self):
+        self.main = torch.cuda.current_stream(self.dev)
+        side = _RoundStreams._side.setdefault(str(self.dev), [])
+        while len(side) < self.n - 1:
+            side.append(torch.cuda.Stream(self.dev))
+        self.streams = [self.main] + side[:self.n - 1]
+        start = self.main.record_event()
+        for s in self.streams[1:]:
+            s.wait_event(start)
+        return self
+
+    def stream(self, i):
+        return torch.cuda.stream(self.streams[i % self.n])
+
+    def __exit__(self, *exc):
+        for s in self.streams[1:]:
+            self.main.wait_event(s.record_event())
+        return False
 
 
 def _cap_windows(windows, nbytes_of_rows, cap):
@@ -179,7 +221,8 @@ def _cap_windows(windows, nbytes_of_rows, cap):
 
 def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engine,
                    bias_func=None, local_bias_args=[], remote_bias_args=[], no_overlap=False, *,
-                   rounds: Optional[int] = None, mask: Optional[Mask] = None, batched: bool = False):
+                   rounds: Optional[int] = None, mask: Optional[Mask] = None, batched: bool = False,
+                   streams: int = 1):
     """Returns (dq, dk, dv) like the reference (attn.py:545): dq [B,Hq,Lq,D];
     dk, dv [B,Hkv,Lkv,D]-shaped views of [B,Lkv,Hkv,D] memory, at the Hkv heads
     k and v came in with.  `o` and `L` are the finally merged forward results;
@@ -187,7 +230,9 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     (attn.py:465-468, 509-527).  dK, dV are summed in fp32 across the q heads of
     a group and across rounds and rounded to bf16 once; a round's dQ rows are
     complete after that round (fp32 sum over all local tokens, rounded once).
-    `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored."""
+    `backward_engine`, `comm_mode`, `no_overlap` are accepted and ignored.  `streams` as in
+    `_attn_forward`; every stream sums its rounds' dK, dV in an fp32 accumulator of its own and
+    the accumulators are added before the one rounding."""
     _reject_unsupported(causal)
     D_in = q.shape[-1]
     q_, k_, v_, o_, do_ = (_usable(_pad_head_dim(t)) for t in (q, k, v, o, do))
@@ -215,17 +260,37 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
         ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk, dv, sm_scale, r0, r1 - r0, mask, accumulate_dkv=False,
                 workspace=ws, bias=bias)
     else:
-        dk_acc = workspace("bwd_dk_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
-        dv_acc = workspace("bwd_dv_acc", (B, Lkv, Hkv, D), torch.float32, dev).transpose(1, 2)
-        dk_acc.zero_()
-        dv_acc.zero_()
-        for r0, r1 in windows:
+        def accumulators():
+            a = workspace("bwd_dkv_acc", (2, B, Lkv, Hkv, D), torch.float32, dev)
+            a.zero_()
+            return a
+
+        def one_round(r0, r1, acc, ws_r):
             ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
-            ops.bwd(q_, k_, v_, do_, L_, delta, dq, dk_acc, dv_acc, sm_scale, r0, r1 - r0, mask,
-                    accumulate_dkv=True, workspace=ws, bias=bias)
+            ops.bwd(q_, k_, v_, do_, L_, delta, dq, acc[0].transpose(1, 2), acc[1].transpose(1, 2), sm_scale,
+                    r0, r1 - r0, mask, accumulate_dkv=True, workspace=ws_r, bias=bias)
+
+        acc = accumulators()
+        n_streams = min(streams, len(windows))
+        if n_streams > 1:
+            ws_bytes = ws.numel()
+            with _RoundStreams(dev, n_streams) as rs:
+                accs = [acc]
+                for j in range(1, n_streams):
+                    with rs.stream(j):
+                        accs.append(accumulators())      # cached per stream, like the dS^T workspace
+                for i, (r0, r1) in enumerate(windows):
+                    with rs.stream(i):
+                        ws_i = ws if i % n_streams == 0 else workspace("bwd_ds", (ws_bytes,), torch.uint8, dev)
+                        one_round(r0, r1, accs[i % n_streams], ws_i)
+            for other in accs[1:]:
+                acc += other
+        else:
+            for r0, r1 in windows:
+                one_round(r0, r1, acc, ws)
         # [B,Hkv,Lkv,D] views of [B,Lkv,Hkv,D] memory: cast in memory order
-        ops.cast_f32(dk_acc.transpose(1, 2), dk.transpose(1, 2))
-        ops.cast_f32(dv_acc.transpose(1, 2), dv.transpose(1, 2))
+        ops.cast_f32(acc[0], dk.transpose(1, 2))
+        ops.cast_f32(acc[1], dv.transpose(1, 2))
     if D_in != D:
         dq = dq[..., :D_in].contiguous()
         dk = dk.transpose(1, 2)[..., :D_in].contiguous().transpose(1, 2)

@@ -377,6 +377,35 @@ def test_backward_cfg1s(lvx, batched):
     check_grad(dv, ref["dv"], "dV")
 
 
+@pytest.mark.parametrize("name", ["cfg1s", "cfg4s"])
+def test_rounds_spread_over_streams(lvx, name):
+    """The rounds of a call touch disjoint rows; queued on three streams instead of one they give
+    the same O, LSE and dQ bit for bit, and dK / dV up to the order of the fp32 sums."""
+    w = orc.make_inputs(orc.workload(name))
+    t = w.tensors
+    ref = orc.layer_reference(w)
+    q, k, v, do = (_dev(t[n]) for n in ("q", "k", "v", "do"))
+    mask = _mask_of(w, lvx)
+    acc = (torch.zeros_like(q), torch.full((w.B * w.Hq, w.Lq), float("-inf"), device=DEV))
+    res = []
+    for n in (1, 3):
+        _, _, _, o, L = lvx._attn_forward(q, k, v, False, w.scale, None, rounds=w.rounds, mask=mask, acc_in=acc,
+                                          streams=n)
+        dq, dk, dv = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash", rounds=w.rounds, mask=mask,
+                                        streams=n)
+        torch.cuda.synchronize()
+        res.append((o, L, dq, dk, dv))
+    (o1, l1, dq1, dk1, dv1), (o3, l3, dq3, dk3, dv3) = res
+    assert torch.equal(o1, o3) and torch.equal(l1, l3) and torch.equal(dq1, dq3)
+    check_o(o3, ref["o"])
+    check_lse(l3, ref["lse"])
+    check_grad(dq3, ref["dq"], "dQ")
+    check_grad(dk3, ref["dk"], "dK")
+    check_grad(dv3, ref["dv"], "dV")
+    for a, b_ in ((dk1, dk3), (dv1, dv3)):
+        assert (a.float() - b_.float()).abs().max() <= 1e-2 * a.float().abs().max()
+
+
 def test_backward_in_row_chunks_under_a_small_workspace_cap(lvx):
     """A window whose dS^T workspace would exceed the cap runs as several calls over row chunks
     (fp32 dK / dV across them): same gradients as the single call."""
