@@ -202,6 +202,8 @@ def run_only(layer, which, n, torch):
         torch.cuda.synchronize()
         print(json.dumps({"only": which, "launches": n, "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
+    if which in ("kv_proj", "dx_vis") and not layer.has_proj:
+        sys.exit(f"bench.py: {w.name} has no K/V projection (Dm = 0)")
     k, v = layer.project()
     B, Hq, Lq, D = layer.q.shape
     Hkv, Lkv = k.shape[1], k.shape[2]

@@ -293,7 +293,8 @@ static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
     return (size_t)2 * s->B * s->Lkv * s->Hkv * s->D * sizeof(float);
 }
 
-// The dQ GEMM of a small row window (a one-round launch) has only B*Hq C tiles; its
+// The dQ GEMM of a small row window (a one-round launch, or few rows against many tokens) has
+// fewer C tiles than the chip has compute units; its
 // contraction over the tokens is then split over several work-groups that store fp32
 // partial tiles, each split into its own slice of a scratch; the slices are summed and
 // rounded to bf16 afterwards (fp32 atomics into one slice were measured slower).  Returns
@@ -304,7 +305,7 @@ static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_le
     const int wgs = s->B * s->Hq * tiles;
     const int blocks = (s->Lkv + 127) / 128;
     int ks = 1;
-    if (wgs < 128) ks = std::min(std::min(8, 256 / wgs), blocks);
+    if (wgs <= 128) ks = std::min(std::min(8, 256 / wgs), blocks);
     const int per = (blocks + ks - 1) / ks;
     *split_len = per * 128;
     return (blocks + per - 1) / per;
