@@ -262,8 +262,16 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
 // Work-groups of the backward are long (every step of a token block) and one
 // fits a CU, so a grid that is not a multiple of the CU count wastes up to one
 // whole round.  Splitting the steps of every token block over `S` work-groups
-// (which then add their dK/dV with atomics) evens that out; S is chosen to
-// minimise ceil(blocks * S / CUs) / S with ranges of at least 32 steps.
+// (which then add their dK/dV with atomics into an fp32 scratch that is zeroed before
+// and rounded after) evens that out.  S minimises
+//     rounds(S) * (steps / S + WG_COST) + (S > 1 ? SPLIT_COST : 0)        [in steps]
+// with ranges of at least 32 steps; WG_COST is what a work-group spends outside its
+// steps (operand load, ring fill, epilogue: about 8 us = 6 steps), SPLIT_COST the zero-fill, the
+// two casts and the slower atomic epilogue (about 70 us).  rounds(S) = ceil(blocks * S / CUs)
+// for equal work-groups.  With an interval mask they differ in length (a token block
+// visits only the row tiles that see it; half of them is assumed), the dispatcher fills the tail by
+// itself and rounds(S) is the plain quotient: splitting then rarely pays (cfg4: 0.98 ms
+// with 5 splits, 0.86 ms with none).
 // CUs of the device that is current (the one the caller's stream belongs to), asked for once per device
 static int cu_count() {
     static int cached[MAX_DEVICES];          // 0: not asked yet
@@ -277,14 +285,21 @@ static int cu_count() {
     return n;
 }
 
-static int choose_q_splits(int blocks, int steps) {
+static int choose_q_splits(int blocks, int steps, bool masked) {
+    constexpr double WG_COST = 6.0, SPLIT_COST = 55.0;
     const int n_cu = cu_count();
+    const double work = masked ? 0.5 * steps : (double)steps;
+    auto cost = [&](int S) {
+        const double rounds = masked ? std::max(1.0, (double)blocks * S / n_cu)
+                                     : (double)(((int64_t)blocks * S + n_cu - 1) / n_cu);
+        return rounds * (work / S + WG_COST) + (S > 1 ? SPLIT_COST : 0.0);
+    };
     int best = 1;
-    double best_cost = (double)((blocks + n_cu - 1) / n_cu);
+    double best_cost = cost(1);
     for (int S = 2; S <= 8; ++S) {
         if (steps / S < 32) break;
-        const double cost = (double)(((int64_t)blocks * S + n_cu - 1) / n_cu) / S;
-        if (cost < best_cost * 0.97) { best_cost = cost; best = S; }
+        const double c = cost(S);
+        if (c < best_cost) { best_cost = c; best = S; }
     }
     return best;
 }
@@ -399,7 +414,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     // metadata kernel zeroes them on its way
     const int blocks = s->B * s->Hkv * p.n_kv_blocks;
     const int steps = p.G * (int)(rows / 32);
-    p.q_splits = choose_q_splits(blocks, steps);
+    p.q_splits = choose_q_splits(blocks, steps, s->kv_start != nullptr);
     p.split_steps = (steps + p.q_splits - 1) / p.q_splits;
     p.total_wg = blocks * p.q_splits;
     p.dkv_mode = p.q_splits > 1 ? 2 : (dkv_accumulate ? 1 : 0);
