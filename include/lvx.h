@@ -20,7 +20,9 @@
  *   - [row_begin, row_begin+row_count) selects the text rows one call works on:
  *     one query block of one round, or all of them at once;
  *   - return value: 0 = queued; negative = argument rejected on the host before
- *     anything was launched (LVX_ERR_*); positive = hipError_t of the launch.
+ *     anything was launched (LVX_ERR_*); positive = hipError_t of the launch that
+ *     failed (entry points that are several launches may have queued the earlier ones;
+ *     a stale error of an unrelated earlier HIP call is neither reported nor cleared).
  *     Nothing throws or aborts.  Calls are re-entrant.
  */
 #ifndef LVX_H
