@@ -56,8 +56,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     const int t1 = wid / p.n_row_tiles;
     const int split = t1 % p.nsplit;
     const int t2 = t1 / p.nsplit;
-    const int hg = t2 % p.n_head_groups;
-    const int b = t2 / p.n_head_groups;
+    // samples vary faster than head groups: every XCD (a contiguous range of ids) then gets
+    // work-groups of all samples, and ragged samples do not leave some XCDs idle early
+    const int b = t2 % p.B;
+    const int hg = t2 / p.B;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;

@@ -119,7 +119,11 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     const int t1 = wid / p.tiles_n;
     const int tm = t1 % p.tiles_m;
     const int t2 = t1 / p.tiles_m;
-    const int z = t2 % p.nbatch;
+    // the outer batch index (the sample, where there is one) varies fastest over the ids, so that
+    // every XCD's contiguous id range holds work of all samples (ragged ones differ in length)
+    const int zr = t2 % p.nbatch;
+    const int n_outer = p.nbatch / p.batch_inner;
+    const int z = (zr % n_outer) * p.batch_inner + zr / n_outer;
     const GemmProblem& pr = p.prob[t2 / p.nbatch];
     const int m0 = tm * TM, n0 = tn * TN;
     const int zo = z / p.batch_inner, zi = z % p.batch_inner;
