@@ -316,6 +316,29 @@ def other_workload(name, torch, dev, steps=10, warmup=5):
             rec["lvx_kv_proj"] = {"ms": round(ms, 4), "tflops": round(f["proj"] / ms / 1e9, 1)}
             ms = time_gpu(lambda: ops.dx_vis(dk, dv, layer.wk, layer.wv), steps, warmup, torch)
             rec["lvx_dx_vis"] = {"ms": round(ms, 4), "tflops": round(f["proj"] / ms / 1e9, 1)}
+        if layer.mask is not None:
+            # the same mask as the reference passes it: a dense additive fp32 bias [B, 1, Lq, Lkv] of
+            # 0 / -inf (what the Hugging Face hook hands over), through the dense-bias kernel variants
+            t = w.tensors
+            keys = torch.arange(Lkv, device=dev).view(1, 1, 1, -1)
+            seen = (keys >= t["kv_start"].to(dev).view(B, 1, Lq, 1)) & (keys < t["kv_end"].to(dev).view(B, 1, Lq, 1)) \
+                & (keys < torch.tensor(w.kv_len, device=dev).view(-1, 1, 1, 1))
+            bias = torch.zeros(B, 1, Lq, Lkv, device=dev).masked_fill_(~seen, float("-inf"))
+            del seen, keys
+            hull = ops.bias_hull(layer.q, k, bias)     # what the host loops do with a bias: skip what it masks
+            ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=hull, bias=bias)
+            ops.bwd_preprocess(o_p, layer.do, delta)
+            bws_d = torch.empty(ops.bwd_workspace_bytes(layer.q, k, Lq, hull), dtype=torch.uint8, device=dev)
+            ms_h = time_gpu(lambda: ops.bias_hull(layer.q, k, bias), steps, warmup, torch)
+            ms_f = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, mask=hull, bias=bias), steps, warmup, torch)
+            ms_b = time_gpu(lambda: ops.bwd(layer.q, k, v, layer.do, l_p, delta, dq, dk, dv, w.scale, mask=hull, bias=bias,
+                                            workspace=bws_d), steps, warmup, torch)
+            ms_f0 = time_gpu(lambda: ops.fwd(layer.q, k, v, o_p, l_p, w.scale, bias=bias), steps, warmup, torch)
+            rec["dense_bias_variant"] = {"lvx_bias_hull_ms": round(ms_h, 4), "lvx_fwd_ms": round(ms_f, 4),
+                                         "lvx_bwd_ms": round(ms_b, 4),
+                                         "tflops_live_pairs": round((f["fwd"] + f["bwd"]) / (2 * ms_h + ms_f + ms_b) / 1e9, 1),
+                                         "lvx_fwd_without_hull_ms": round(ms_f0, 4), "bias_bytes": bias.numel() * 4}
+            del bias, bws_d
     del layer, other
     layer = other = None
     from lv_xattn import reset_global_memory_buffer

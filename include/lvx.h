@@ -129,6 +129,18 @@ int lvx_merge(const lvx_attn_shape* shape, const lvx_tensor* o_acc, float* l_acc
               int32_t row_begin, int32_t row_count, void* stream);
 
 /*
+ * kv_start / kv_end [B, Lq] (int32, written): per text row the hull of the keys that
+ * shape->bias leaves visible (entries other than -inf; over all heads when bias_stride_h != 0;
+ * (0, 0) for a row that sees nothing).  Passed back as shape->kv_start / kv_end next to the same
+ * bias, they let lvx_fwd / lvx_bwd skip the tiles outside the hull; the results do not change,
+ * because a bias of -inf removes those pairs anyway.  shape->kv_start / kv_end are not read here.
+ * No counterpart in the reference, which loads and adds its dense bias on every tile of a
+ * block (lv_xattn/attn.py:238-241, flash_attn_kernels.py:496-512): this is the step that makes
+ * a mask handed over as a bias cost what it leaves visible.
+ */
+int lvx_bias_hull(const lvx_attn_shape* shape, int32_t* kv_start, int32_t* kv_end, void* stream);
+
+/*
  * delta[b*Hq+h, row] = sum_d O * dO.  Replaces `_bwd_preprocess_do_o_dot`
  * (lv_xattn/flash_attn_kernels.py:287-329, launched at :926-942).
  */

@@ -241,6 +241,16 @@ int lvx_merge(const lvx_attn_shape* s, const lvx_tensor* o_acc, float* l_acc, co
     return static_cast<int>(launch_merge(m, static_cast<hipStream_t>(stream)));
 }
 
+int lvx_bias_hull(const lvx_attn_shape* s, int32_t* kv_start, int32_t* kv_end, void* stream) {
+    LVX_TRY(check_shape(s));
+    if (!s->bias || !kv_start || !kv_end) return LVX_ERR_NULL;
+    BiasHullParams p{};
+    p.bias = s->bias; p.bias_b = s->bias_stride_b; p.bias_h = s->bias_stride_h; p.bias_r = s->bias_stride_r;
+    p.kv_start = kv_start; p.kv_end = kv_end;
+    p.B = s->B; p.heads = s->bias_stride_h ? s->Hq : 1; p.Lq = s->Lq; p.Lkv = s->Lkv;
+    return static_cast<int>(launch_bias_hull(p, static_cast<hipStream_t>(stream)));
+}
+
 int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_tensor* dout, float* delta,
                        int32_t row_begin, int32_t row_count, void* stream) {
     LVX_TRY(check_shape(s));

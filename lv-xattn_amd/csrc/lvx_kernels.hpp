@@ -59,6 +59,16 @@ struct MergeParams {
     int f16;
 };
 
+// Per text row the hull of the keys a dense bias leaves visible (entries other than -inf).
+struct BiasHullParams {
+    const float* bias;
+    int64_t bias_b, bias_h, bias_r;
+    int32_t* kv_start;         // out [B, Lq]
+    int32_t* kv_end;           // out [B, Lq]
+    int B, heads, Lq, Lkv;     // heads: 1 (bias broadcast over heads) or Hq
+};
+hipError_t launch_bias_hull(const BiasHullParams& p, hipStream_t st);
+
 struct PreParams {
     const uint16_t* o;
     const uint16_t* dout;

@@ -227,6 +227,34 @@ __global__ __launch_bounds__(256) void bwd_meta_kernel(const MetaParams p) {
     o[32] = d * p.scale;
 }
 
+// One wave per (b, text row): first and one-past-last key whose bias is not -inf, over all heads
+// the bias distinguishes.  An empty row gets (0, 0).
+__global__ __launch_bounds__(256) void bias_hull_kernel(const BiasHullParams p) {
+    const int64_t rw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (rw >= (int64_t)p.B * p.Lq) return;
+    const int b = (int)(rw / p.Lq), row = (int)(rw % p.Lq);
+    int lo = INT_MAX, hi = 0;
+    for (int h = 0; h < p.heads; ++h) {
+        const float* br = p.bias + b * p.bias_b + h * p.bias_h + (int64_t)row * p.bias_r;
+        for (int k0 = 4 * lane; k0 < p.Lkv; k0 += 256) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(br + k0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (k0 + j < p.Lkv && !(v[j] == -INFINITY)) { lo = min(lo, k0 + j); hi = max(hi, k0 + j + 1); }
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        lo = min(lo, __shfl_xor(lo, o));
+        hi = max(hi, __shfl_xor(hi, o));
+    }
+    if (lane == 0) {
+        p.kv_start[rw] = hi > 0 ? lo : 0;
+        p.kv_end[rw] = hi;
+    }
+}
+
 // One wave per (group of row tiles, b): the hull of the rows' key intervals in whole token blocks.
 __global__ __launch_bounds__(64) void bwd_hull_kernel(const LiveParams p) {
     const int grp = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
@@ -415,6 +443,12 @@ hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st) {
     const hipError_t e = launch1(bwd_hull_kernel, dim3(p.n_groups, p.B), dim3(64), st, p);
     if (e != hipSuccess) return e;
     return launch1(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), st, p);
+}
+
+hipError_t launch_bias_hull(const BiasHullParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.B * p.Lq;
+    if (rows == 0) return hipSuccess;
+    return launch1(bias_hull_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), st, p);
 }
 
 hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {

@@ -135,6 +135,8 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     bias = _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, k_.shape[2], dev)
     if mask is not None:
         mask = mask.to(dev)
+    elif bias is not None:
+        mask = ops.bias_hull(q_, k_, bias)    # skip what the bias masks out anyway
 
     o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
     L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
@@ -243,6 +245,8 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     bias = _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, dev)
     if mask is not None:
         mask = mask.to(dev)
+    elif bias is not None:
+        mask = ops.bias_hull(q_, k_, bias)    # as in the forward: the same hull, hence the same pairs
     L_ = L.to(torch.float32).reshape(B * Hq, Lq).contiguous()
 
     delta = workspace("bwd_delta", (B * Hq, Lq), torch.float32, dev)

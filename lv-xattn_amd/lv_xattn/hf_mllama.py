@@ -50,8 +50,14 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     there).  The masks transformers builds hold no such row: its
     _prepare_cross_attention_mask multiplies the mask by
     full_text_row_masked_out_mask, which turns a row that sees no tile into a
-    row that sees every key."""
-    return mask.float().clamp_min(-30000.0)
+    row that sees every key.
+    Where a row does see a key, its masked positions become -inf: the result is the same
+    (exp(-30000) is already 0 there) and the kernels can then skip whole tiles outside the span
+    of the visible keys (ops.bias_hull), which is most of a Llama-3.2 mask."""
+    m = mask.float()
+    masked = m <= -30000.0
+    sees_a_key = (~masked).any(-1, keepdim=True)
+    return torch.where(masked & sees_a_key, float("-inf"), m.clamp_min(-30000.0))
 
 
 def lv_xattn_attention_forward(module, query, key, value, attention_mask: Optional[torch.Tensor],

@@ -127,6 +127,19 @@ def merge(o_acc, l_acc, o_part, l_part, row_begin=0, row_count=None) -> None:
     check(rc, "lvx_merge")
 
 
+def bias_hull(q, k, bias: torch.Tensor) -> Mask:
+    """The interval mask a dense bias implies: per text row the hull of its entries other
+    than -inf.  Given to fwd / bwd together with the bias it lets them skip what the bias
+    masks anyway."""
+    s = _shape(q, k, 1.0, None, bias)
+    B, Lq = q.shape[0], q.shape[2]
+    start = torch.empty(B, Lq, dtype=torch.int32, device=q.device)
+    end = torch.empty_like(start)
+    rc = load().lvx_bias_hull(C.byref(s), start.data_ptr(), end.data_ptr(), stream_ptr())
+    check(rc, "lvx_bias_hull")
+    return Mask(None, start, end)
+
+
 def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
     B, Hq, Lq, D = o.shape
     s = AttnShape(B, Hq, Hq, D, Lq, 1, dtype_code(o, dout), 1.0, None, None, None)

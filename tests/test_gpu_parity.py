@@ -617,3 +617,62 @@ def test_dense_bias_forward_backward(lvx, batched):
     check_grad(dv, dv_ref, "dV")
     dead = torch.isinf(l_ref)
     assert dead.any() and (o.float().cpu()[dead] == 0).all() and (dq.float().cpu()[dead] == 0).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("per_head,per_sample", [(False, True), (True, True), (False, False)])
+def test_bias_hull_is_the_span_of_the_finite_entries(lvx, per_head, per_sample):
+    """lvx_bias_hull against torch on a bias with -inf bands, an all -inf row, a row with one
+    visible key and a key length that is not a multiple of 4; with it as the mask, forward and
+    backward give what the dense-bias kernels give alone (the pairs outside the hull are exactly
+    those a -inf bias removes)."""
+    from lv_xattn import ops
+    B, Hq, Hkv, Lq, Lkv, D = 2, 8, 2, 200, 1601, 128
+    g = torch.Generator().manual_seed(5)
+    bias = 0.3 * torch.randn(B if per_sample else 1, Hq if per_head else 1, Lq, Lkv, generator=g)
+    for r in range(Lq):
+        lo, hi = (r * 7) % 900, 901 + (r * 13) % 700
+        bias[:, :, r, :lo] = float("-inf")
+        bias[:, :, r, hi:] = float("-inf")
+    if per_head:
+        bias[:, 3, :, 100:300] = 0.25          # one head sees further to the left
+    bias[:, :, 17, :] = float("-inf")
+    bias[:, :, 18, :] = float("-inf")
+    bias[:, :, 18, 1600] = 0.0
+    bias[:, :, :, 400:500:3] = float("-inf")   # holes inside the hull stay the bias's business
+    pad = torch.zeros(*bias.shape[:3], Lkv + 3)
+    pad[..., :Lkv] = bias
+    bias_d = pad.to(DEV)[..., :Lkv]
+    q = (torch.randn(B, Hq, Lq, D, generator=g)).to(torch.bfloat16).to(DEV)
+    k = (torch.randn(B, Hkv, Lkv, D, generator=g)).to(torch.bfloat16).to(DEV)
+    v = (torch.randn(B, Hkv, Lkv, D, generator=g)).to(torch.bfloat16).to(DEV)
+    do = (torch.randn(B, Hq, Lq, D, generator=g)).to(torch.bfloat16).to(DEV)
+    m = ops.bias_hull(q, k, bias_d)
+    live = ~torch.isinf(bias.expand(B, bias.shape[1], Lq, Lkv)).all(1) if per_head else ~torch.isinf(bias.expand(B, 1, Lq, Lkv))[:, 0]
+    idx = torch.arange(Lkv).view(1, 1, -1)
+    want_s = torch.where(live, idx, Lkv).amin(-1)
+    want_e = torch.where(live, idx + 1, 0).amax(-1)
+    want_s = torch.where(want_e > 0, want_s, 0)
+    assert torch.equal(m.kv_start.cpu(), want_s.to(torch.int32)) and torch.equal(m.kv_end.cpu(), want_e.to(torch.int32))
+
+    scale = D ** -0.5
+    outs = []
+    for mask in (None, m):
+        o, L = torch.empty_like(q), torch.empty(B * Hq, Lq, device=DEV)
+        ops.fwd(q, k, v, o, L, scale, mask=mask, bias=bias_d)
+        delta = torch.empty_like(L)
+        ops.bwd_preprocess(o, do, delta)
+        dq = torch.empty_like(q)
+        dk = torch.empty(B, Lkv, Hkv, D, dtype=torch.bfloat16, device=DEV).transpose(1, 2)
+        dv = torch.empty_like(dk.transpose(1, 2)).transpose(1, 2)
+        ws = torch.empty(ops.bwd_workspace_bytes(q, k, Lq, mask), dtype=torch.uint8, device=DEV)
+        ops.bwd(q, k, v, do, L, delta, dq, dk, dv, scale, mask=mask, workspace=ws, bias=bias_d)
+        outs.append((o, L, dq, dk, dv))
+    torch.cuda.synchronize()
+    (o0, L0, dq0, dk0, dv0), (o1, L1, dq1, dk1, dv1) = outs
+    assert torch.equal(torch.isinf(L0), torch.isinf(L1)) and torch.isinf(L0).any()
+    fin = ~torch.isinf(L0)
+    assert (L0[fin] - L1[fin]).abs().max() <= 1e-5
+    for a, b_, what in ((o0, o1, "O"), (dq0, dq1, "dQ"), (dk0, dk1, "dK"), (dv0, dv1, "dV")):
+        ref = a.float().abs().max()
+        assert (a.float() - b_.float()).abs().max() <= 4e-3 * ref, what
