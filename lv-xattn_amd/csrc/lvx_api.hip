@@ -279,9 +279,9 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
 // steps (operand load, ring fill, epilogue: about 8 us = 6 steps), SPLIT_COST the zero-fill, the
 // two casts and the slower atomic epilogue (about 70 us).  rounds(S) = ceil(blocks * S / CUs)
 // for equal work-groups.  With an interval mask they differ in length (a token block
-// visits only the row tiles that see it; half of them is assumed), the dispatcher fills the tail by
-// itself and rounds(S) is the plain quotient: splitting then rarely pays (cfg4: 0.98 ms
-// with 5 splits, 0.86 ms with none).
+// visits only the row tiles that see it; half of them is assumed); given at least two per CU the
+// dispatcher fills the tail by itself and rounds(S) is the plain quotient: splitting then
+// rarely pays (cfg4: 0.98 ms with 5 splits, 0.86 ms with none).
 // CUs of the device that is current (the one the caller's stream belongs to), asked for once per device
 static int cu_count() {
     static int cached[MAX_DEVICES];          // 0: not asked yet
@@ -298,9 +298,12 @@ static int cu_count() {
 static int choose_q_splits(int blocks, int steps, bool masked) {
     constexpr double WG_COST = 6.0, SPLIT_COST = 55.0;
     const int n_cu = cu_count();
-    const double work = masked ? 0.5 * steps : (double)steps;
+    // unequal work-groups only even out when there are enough of them; a small masked launch
+    // is priced like a dense one (which is also right when its mask hides nothing)
+    const bool ragged = masked && blocks >= 2 * n_cu;
+    const double work = ragged ? 0.5 * steps : (double)steps;
     auto cost = [&](int S) {
-        const double rounds = masked ? std::max(1.0, (double)blocks * S / n_cu)
+        const double rounds = ragged ? (double)blocks * S / n_cu
                                      : (double)(((int64_t)blocks * S + n_cu - 1) / n_cu);
         return rounds * (work / S + WG_COST) + (S > 1 ? SPLIT_COST : 0.0);
     };
