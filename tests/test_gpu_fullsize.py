@@ -202,3 +202,45 @@ def test_full_size_runs_repeat_bit_for_bit(lvx, name, batched):
                                b.view(torch.int16 if b.dtype != torch.float32 else torch.int32)), what
         for a, b, what in zip(cur[3:], first[3:], ("dK", "dV")):
             assert (a - b).abs().max().item() <= 2e-2 * b.abs().max().item(), what
+
+
+def test_eight_samples_of_cfg2_shape_with_the_backward_cut_by_the_workspace_cap(lvx):
+    """B = 8 at cfg2's shape (the backward's dS^T workspace would be 13.7 GB): the default cap
+    cuts the window into two calls, a 4 GiB cap into four; all give the same gradients to
+    rounding, and a sample computed in the batch equals the same sample computed alone (O, LSE and
+    dQ bit for bit: nothing that writes them depends on the batch or uses atomics)."""
+    from lv_xattn.async_communication import (backward_workspace_cap, reset_global_memory_buffer,
+                                              set_backward_workspace_cap)
+    B, Hq, Hkv, D, Lq, Lkv, P = 8, 32, 8, 128, 4096, 6404, 16
+    g = torch.Generator().manual_seed(8)
+    rn = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)
+    q, do = rn(B, Hq, Lq, D), rn(B, Hq, Lq, D)
+    k, v = rn(B, Lkv, Hkv, D).transpose(1, 2), rn(B, Lkv, Hkv, D).transpose(1, 2)
+    scale = D ** -0.5
+    _, _, _, o, L = lvx._attn_forward(q, k, v, False, scale, None, rounds=P, batched=True)
+    old_cap = backward_workspace_cap()
+    grads = []
+    try:
+        for cap_gib in (16, 12, 4):
+            set_backward_workspace_cap(cap_gib << 30)
+            reset_global_memory_buffer()
+            torch.cuda.empty_cache()
+            grads.append(tuple(t.clone() for t in lvx._attn_backward(do, q, k, v, o, L, False, scale, None, "flash",
+                                                                     rounds=P, batched=True)))
+        torch.cuda.synchronize()
+    finally:
+        set_backward_workspace_cap(old_cap)
+        reset_global_memory_buffer()
+    for other in grads[1:]:
+        for a, b_, what in zip(grads[0], other, ("dQ", "dK", "dV")):
+            assert (a.float() - b_.float()).abs().max() <= 4e-3 * a.float().abs().max(), what
+    b = 5
+    one = lambda t: t[b:b + 1].contiguous() if t.is_contiguous() else t[b:b + 1]
+    _, _, _, o1, L1 = lvx._attn_forward(one(q), k[b:b + 1], v[b:b + 1], False, scale, None, rounds=P, batched=True)
+    dq1, dk1, dv1 = lvx._attn_backward(one(do), one(q), k[b:b + 1], v[b:b + 1], o1, L1, False, scale, None, "flash",
+                                       rounds=P, batched=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o1[0], o[b]) and torch.equal(L1.view(Hq, Lq), L.view(B, Hq, Lq)[b])
+    assert torch.equal(dq1[0], grads[0][0][b])
+    for a, b_, what in ((dk1[0], grads[0][1][b], "dK"), (dv1[0], grads[0][2][b], "dV")):
+        assert (a.float() - b_.float()).abs().max() <= 4e-3 * a.float().abs().max(), what
