@@ -339,12 +339,52 @@ def other_workload(name, torch, dev, steps=10, warmup=5):
                                          "tflops_live_pairs": round((f["fwd"] + f["bwd"]) / (2 * ms_h + ms_f + ms_b) / 1e9, 1),
                                          "lvx_fwd_without_hull_ms": round(ms_f0, 4), "bias_bytes": bias.numel() * 4}
             del bias, bws_d
+            rec["hf_attention_interface"] = hf_interface_time(layer, k, v, seen_mask=None, w=w, f=f, steps=steps,
+                                                              warmup=warmup, torch=torch, dev=dev)
     del layer, other
     layer = other = None
     from lv_xattn import reset_global_memory_buffer
     reset_global_memory_buffer()
     torch.cuda.empty_cache()
     return rec
+
+
+def hf_interface_time(layer, k, v, seen_mask, w, f, steps, warmup, torch, dev):
+    """Forward + backward through the Hugging Face attention-interface function with the mask as
+    transformers hands it over: additive [B, 1, Lq, Lkv] in the model's element type, the type's
+    most negative finite value where masked.  Includes the mask's conversion to the fp32 bias
+    (torch element-wise passes), the hull kernel and the autograd wrapper."""
+    try:
+        from lv_xattn import hf_mllama
+    except Exception as e:          # transformers missing or too old: no such path to time
+        return {"skipped": type(e).__name__}
+    t = w.tensors
+    B, Hq, Lq, D = layer.q.shape
+    Lkv = k.shape[2]
+    keys = torch.arange(Lkv, device=dev).view(1, 1, 1, -1)
+    seen = (keys >= t["kv_start"].to(dev).view(B, 1, Lq, 1)) & (keys < t["kv_end"].to(dev).view(B, 1, Lq, 1)) \
+        & (keys < torch.tensor(w.kv_len, device=dev).view(-1, 1, 1, 1))
+    attn_mask = torch.zeros(B, 1, Lq, Lkv, dtype=w.dtype, device=dev).masked_fill_(~seen, torch.finfo(w.dtype).min)
+    # rows that see nothing: transformers turns them into rows that see everything
+    attn_mask = attn_mask * seen.any(-1, keepdim=True).to(w.dtype)
+    del seen, keys
+
+    class _Module:            # what the function reads of the attention module
+        is_causal = False
+        k_norm = None
+
+    q = layer.q.detach().clone().requires_grad_(True)
+    kk, vv = k.detach().clone().requires_grad_(True), v.detach().clone().requires_grad_(True)
+    do_t = layer.do.transpose(1, 2).contiguous()
+
+    def run():
+        out, _ = hf_mllama.lv_xattn_attention_forward(_Module(), q, kk, vv, attn_mask, dropout=0.0, scaling=w.scale)
+        out.backward(do_t)
+        q.grad = kk.grad = vv.grad = None
+
+    ms = time_gpu(run, steps, warmup, torch)
+    return {"fwd_bwd_ms": round(ms, 4), "tflops_live_pairs": round((f["fwd"] + f["bwd"]) / ms / 1e9, 1),
+            "mask": f"{w.dtype} additive [B,1,Lq,Lkv], finfo.min where masked"}
 
 
 def cpu_baseline(w, budget_rounds=8):

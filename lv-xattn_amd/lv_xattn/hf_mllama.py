@@ -37,6 +37,7 @@ from .autograd import create_attention_class, create_attention_class_save_qkv, c
 
 NAME = "lv_xattn"
 _attention = None
+_bias_cache: list = []      # [key, fp32 bias, the mask it was made from] of the last conversion
 
 
 def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
@@ -54,10 +55,17 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     Where a row does see a key, its masked positions become -inf: the result is the same
     (exp(-30000) is already 0 there) and the kernels can then skip whole tiles outside the span
     of the visible keys (ops.bias_hull), which is most of a Llama-3.2 mask."""
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
+    if _bias_cache and _bias_cache[0] == key:
+        return _bias_cache[1]
     m = mask.float()
     masked = m <= -30000.0
     sees_a_key = (~masked).any(-1, keepdim=True)
-    return torch.where(masked & sees_a_key, float("-inf"), m.clamp_min(-30000.0))
+    bias = torch.where(masked & sees_a_key, float("-inf"), m.clamp_min(-30000.0))
+    # every cross-attention layer of a model gets the same mask, in forward and again in backward:
+    # the last conversion is kept (with the mask itself, so that its address cannot be reused)
+    _bias_cache[:] = [key, bias, mask]
+    return bias
 
 
 def lv_xattn_attention_forward(module, query, key, value, attention_mask: Optional[torch.Tensor],
