@@ -97,6 +97,18 @@ int lvx_fwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* 
             int32_t row_begin, int32_t row_count, int32_t kv_splits,
             void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * lvx_fwd whose result is merged with an incoming accumulator (o_in [like o], l_in
+ * [B*Hq, Lq], only read) before it is written to (o, lse): one round's _fwd_kernel launch plus
+ * its _rescale_kernel launch (lv_xattn/attn.py:390-400 and 403-419) in one call.  With key
+ * splits the partials and the accumulator are folded by the same merge launch; o must not be
+ * o_in (LVX_ERR_SHAPE).  Workspace as for lvx_fwd.
+ */
+int lvx_fwd_acc(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+                const lvx_tensor* o_in, const float* l_in, const lvx_tensor* o, float* lse,
+                int32_t row_begin, int32_t row_count, int32_t kv_splits,
+                void* workspace, size_t workspace_bytes, void* stream);
+
 size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* shape, int32_t row_count, int32_t kv_splits);
 
 /*

@@ -120,9 +120,11 @@ size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count, int32
     return (size_t)kv_splits * rows * (s->D * sizeof(uint16_t) + sizeof(float));
 }
 
-int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
-            const lvx_tensor* o, float* lse, int32_t row_begin, int32_t row_count, int32_t kv_splits,
-            void* workspace, size_t workspace_bytes, void* stream) {
+// lvx_fwd, and lvx_fwd_acc when (o_in, l_in) is given: the result is then merged with that
+// incoming accumulator before it is written to (o, lse).
+static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+                    const lvx_tensor* o, float* lse, int32_t row_begin, int32_t row_count, int32_t kv_splits,
+                    void* workspace, size_t workspace_bytes, void* stream, const lvx_tensor* o_in, const float* l_in) {
     LVX_TRY(check_shape(s));
     LVX_TRY(check_tensor(q));
     LVX_TRY(check_tensor(k));
@@ -163,7 +165,25 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         p.os = st3(o);
         p.lse = lse;
         p.lse_bh_stride = s->Lq;
-        return static_cast<int>(launch_fwd(p, s->kv_start != nullptr, st));
+        const hipError_t e1 = launch_fwd(p, s->kv_start != nullptr, st);
+        if (e1 != hipSuccess || !o_in) return static_cast<int>(e1);
+        // one partial, written straight to (o, lse): fold the incoming accumulator into it (the
+        // merge is symmetric, so which side is "the accumulator" does not matter)
+        MergeParams m{};
+        m.f16 = s->dtype == LVX_F16;
+        m.o_acc = static_cast<uint16_t*>(o->ptr);
+        m.l_acc = lse;
+        m.o_part = static_cast<const uint16_t*>(o_in->ptr);
+        m.l_part = l_in;
+        m.oa = st3(o);
+        m.op = st3(o_in);
+        m.l_acc_bh = s->Lq;
+        m.l_part_bh = s->Lq;
+        m.nparts = 1;
+        m.use_acc = 1;
+        m.B = s->B; m.Hq = s->Hq; m.Lq = s->Lq;
+        m.row_begin = row_begin; m.row_end = row_begin + row_count;
+        return static_cast<int>(launch_merge(m, st));
     }
 
     // key splits: partials [split][B*Hq][row_count][D] + LSE [split][B*Hq][row_count]
@@ -197,9 +217,34 @@ int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     m.l_part_bh = row_count;
     m.nparts = nsplit;
     m.use_acc = 0;
+    if (o_in) {      // the partials and the incoming accumulator in one launch
+        m.use_acc = 1;
+        m.o_in = static_cast<const uint16_t*>(o_in->ptr);
+        m.l_in = l_in;
+        m.oi = st3(o_in);
+        m.l_in_bh = s->Lq;
+    }
     m.B = s->B; m.Hq = s->Hq; m.Lq = s->Lq;
     m.row_begin = row_begin; m.row_end = row_begin + row_count;
     return static_cast<int>(launch_merge(m, st));
+}
+
+int lvx_fwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+            const lvx_tensor* o, float* lse, int32_t row_begin, int32_t row_count, int32_t kv_splits,
+            void* workspace, size_t workspace_bytes, void* stream) {
+    return fwd_impl(s, q, k, v, o, lse, row_begin, row_count, kv_splits, workspace, workspace_bytes, stream,
+                    nullptr, nullptr);
+}
+
+int lvx_fwd_acc(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
+                const lvx_tensor* o_in, const float* l_in, const lvx_tensor* o, float* lse, int32_t row_begin,
+                int32_t row_count, int32_t kv_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!o_in) return LVX_ERR_NULL;
+    LVX_TRY(check_tensor(o_in));
+    if (!l_in) return LVX_ERR_NULL;
+    if (o && o_in->ptr == o->ptr) return LVX_ERR_SHAPE;     // the result is formed out of place
+    return fwd_impl(s, q, k, v, o, lse, row_begin, row_count, kv_splits, workspace, workspace_bytes, stream,
+                    o_in, l_in);
 }
 
 size_t lvx_noalloc_scratch_bytes(void) { return NOALLOC_SCRATCH_BYTES; }

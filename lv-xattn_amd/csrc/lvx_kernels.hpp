@@ -55,6 +55,12 @@ struct MergeParams {
     int64_t l_acc_bh, l_part_bh;
     int nparts;
     int use_acc;               // 1: fold into the existing accumulator, 0: overwrite
+    // with use_acc and several parts: where the accumulator is read from when it is not
+    // (o_acc, l_acc) itself, which then only receive the result (null: in place)
+    const uint16_t* o_in;
+    const float* l_in;
+    Strides3 oi;
+    int64_t l_in_bh;
     int B, Hq, Lq, row_begin, row_end;
     int f16;
 };

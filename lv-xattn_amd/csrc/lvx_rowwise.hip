@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     const int b = bh / p.Hq, h = bh % p.Hq;
 
     float la = -INFINITY;
-    if (p.use_acc) la = p.l_acc[(int64_t)bh * p.l_acc_bh + row];
+    if (p.use_acc) la = p.l_in ? p.l_in[(int64_t)bh * p.l_in_bh + row] : p.l_acc[(int64_t)bh * p.l_acc_bh + row];
     float lp[MAX_PARTS];
     float m = la;
 #pragma unroll
@@ -67,7 +67,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     uint16_t* oa = p.o_acc + b * p.oa.b + h * p.oa.h + (int64_t)row * p.oa.s + chunk * 8;
     if (p.use_acc) {
         float f[8];
-        unpack8<E>(*reinterpret_cast<const u32x4*>(oa), f);
+        const uint16_t* oin = p.o_in ? p.o_in + b * p.oi.b + h * p.oi.h + (int64_t)row * p.oi.s + chunk * 8 : oa;
+        unpack8<E>(*reinterpret_cast<const u32x4*>(oin), f);
         const float w = wa * inv;
         // an accumulator with weight 0 (L = -inf: nothing folded in yet) may hold anything
         if (w > 0.f) {
@@ -412,7 +413,7 @@ inline int blocks_for(int64_t rows) { return (int)((rows * 16 + 255) / 256); }
 hipError_t launch_merge(const MergeParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Hq * (p.row_end - p.row_begin);
     if (rows == 0) return hipSuccess;
-    if (p.nparts == 1 && p.use_acc) {
+    if (p.nparts == 1 && p.use_acc && !p.o_in) {
         const dim3 grid(blocks_for((rows + 1) / 2));
         if (p.f16) return launch1(merge_pair_kernel<true>, grid, dim3(256), st, p);
         return launch1(merge_pair_kernel<false>, grid, dim3(256), st, p);

@@ -44,6 +44,7 @@ SYMBOLS = {
     "lvx_strerror": (C.c_char_p, [C.c_int]),
     "lvx_fwd_workspace_bytes": (C.c_size_t, [_SHAPE, C.c_int32, C.c_int32]),
     "lvx_fwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, C.c_int32, C.c_int32, C.c_int32, _P, C.c_size_t, _P]),
+    "lvx_fwd_acc": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, _T, _P, C.c_int32, C.c_int32, C.c_int32, _P, C.c_size_t, _P]),
     "lvx_fwd_noalloc": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, C.c_int32, C.c_int32, C.c_int32, _P]),
     "lvx_noalloc_scratch_bytes": (C.c_size_t, []),
     "lvx_merge": (C.c_int, [_SHAPE, _T, _P, _T, _P, C.c_int32, C.c_int32, _P]),

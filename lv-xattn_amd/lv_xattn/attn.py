@@ -153,13 +153,13 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
         nbytes = ops.fwd_workspace_bytes(q_, k_, max_rows, kv_splits)
         ws = workspace("fwd_split", (nbytes,), torch.uint8, dev)
 
-    # the partial goes straight into (o, L); an incoming accumulator is then folded into it
-    # (the merge is symmetric, so which side is "the accumulator" does not matter, and neither
-    # a copy of acc_in nor a buffer for the partial is needed)
+    # the partial goes straight into (o, L), merged on its way with the incoming accumulator
+    # if there is one (with key splits by the launch that folds the splits; neither a copy of
+    # acc_in nor a buffer for the partial is needed)
+    acc = (acc_o, acc_l) if acc_in is not None else None
+
     def one_round(r0, r1, ws):
-        ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias)
-        if acc_in is not None:
-            ops.merge(o, L, acc_o, acc_l, r0, r1 - r0)
+        ops.fwd(q_, k_, v_, o, L, sm_scale, r0, r1 - r0, mask, kv_splits, ws, bias, acc=acc)
 
     if streams > 1 and len(windows) > 1:
         with _RoundStreams(dev, min(streams, len(windows))) as rs:

@@ -82,15 +82,27 @@ def fwd_workspace_bytes(q, k, row_count: int, kv_splits: int) -> int:
 
 
 def fwd(q, k, v, o, lse, scale, row_begin=0, row_count=None, mask: Optional[Mask] = None,
-        kv_splits: int = 1, workspace: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
+        kv_splits: int = 1, workspace: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+        acc=None) -> None:
     """Partial O (bf16) and LSE (fp32 [B*Hq, Lq]) of text rows
     [row_begin, row_begin+row_count) against the whole local K/V shard.
-    `bias`: dense additive fp32 [B|1, Hq|1, Lq, Lkv], added after the scale."""
+    `bias`: dense additive fp32 [B|1, Hq|1, Lq, Lkv], added after the scale.
+    `acc` = (o_in like o, l_in fp32 [B*Hq, Lq]): an incoming accumulator the result is merged
+    with before it is written (lvx_fwd_acc); only read, and not o itself."""
     s = _shape(q, k, scale, mask, bias)
     if row_count is None:
         row_count = q.shape[2] - row_begin
     _check_lse(lse, q)
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    if acc is not None:
+        o_in, l_in = acc
+        dtype_code(q, o_in)
+        _check_lse(l_in, q)
+        rc = load().lvx_fwd_acc(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(o_in)),
+                                l_in.data_ptr(), C.byref(t4(o)), lse.data_ptr(), row_begin, row_count, kv_splits,
+                                ws_ptr, ws_bytes, stream_ptr())
+        check(rc, "lvx_fwd_acc")
+        return
     rc = load().lvx_fwd(C.byref(s), C.byref(t4(q)), C.byref(t4(k)), C.byref(t4(v)), C.byref(t4(o)),
                         lse.data_ptr(), row_begin, row_count, kv_splits, ws_ptr, ws_bytes, stream_ptr())
     check(rc, "lvx_fwd")

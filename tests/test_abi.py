@@ -103,6 +103,18 @@ def test_other_entry_points_reject_bad_arguments(lib):
     assert lib.lvx_merge(C.byref(s), C.byref(t), 0x2000, C.byref(t), 0x2000, 0, 65, None) == -3
     assert lib.lvx_bwd_preprocess(C.byref(s), C.byref(t), C.byref(_t(ptr=8)), 0x2000, 0, 64, None) == -2
     assert lib.lvx_bias_hull(C.byref(s), 0x2000, 0x3000, None) == -1          # a shape without a bias
+    # lvx_fwd_acc: the accumulator must be there, aligned, and not the output itself
+    o_in = _t(ptr=0x9000)
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), None, 0x2000, C.byref(t), 0x2000,
+                           0, 64, 1, None, 0, None) == -1
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(o_in), None, C.byref(t), 0x2000,
+                           0, 64, 1, None, 0, None) == -1
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(_t(ptr=8)), 0x2000, C.byref(t),
+                           0x2000, 0, 64, 1, None, 0, None) == -2
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, C.byref(t), 0x2000,
+                           0, 64, 1, None, 0, None) == -3
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(o_in), 0x2000, C.byref(t), 0x2000,
+                           0, 0, 1, None, 0, None) == 0          # no rows: accepted, nothing launched
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, None, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, 1 << 30, None) == -1
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),

@@ -282,19 +282,32 @@ def test_forward_cfg1s(lvx, mode):
     check_lse(L, l_ref)
 
 
-def test_forward_with_incoming_accumulator(lvx):
+@pytest.mark.parametrize("kw", [dict(), dict(kv_splits=1), dict(kv_splits=4), dict(batched=True),
+                                dict(batched=True, kv_splits=3)],
+                         ids=["auto", "nosplit", "split4", "batched", "batched_split3"])
+def test_forward_with_incoming_accumulator(lvx, kw):
+    # lvx_fwd_acc: the round's partial and the travelling accumulator leave as one result; with
+    # key splits one merge launch folds the splits and the accumulator, which may hold NaN
+    # where its LSE is -inf (nothing folded in yet)
     w = orc.make_inputs(orc.workload("cfg1s"))
     t = w.tensors
     g = torch.Generator().manual_seed(11)
     o_in = torch.randn(w.B, w.Hq, w.Lq, w.D, generator=g).bfloat16()
     l_in = torch.randn(w.B, w.Hq, w.Lq, generator=g) * 0.1 + math.log(w.Lkv) + 0.5
+    l_in[:, :, 5::17] = float("-inf")
+    o_clean = o_in.clone()
+    o_clean[l_in.isinf()] = 0
+    o_in[l_in.isinf()] = float("nan")
     o_ref, l_ref = orc.round_loop_forward(t["q"], t["k"], t["v"], w.scale, w.rounds,
-                                          acc_in=(o_in, l_in), round_to_bf16=True)
+                                          acc_in=(o_clean, l_in), round_to_bf16=True)
+    o_d, l_d = _dev(o_in), _dev(l_in)
     _, _, _, o, L = lvx._attn_forward(_dev(t["q"]), _dev(t["k"]), _dev(t["v"]), False, w.scale, None,
-                                      rounds=w.rounds, acc_in=(_dev(o_in), _dev(l_in)))
+                                      rounds=w.rounds, acc_in=(o_d, l_d), **kw)
     torch.cuda.synchronize()
     check_o(o, o_ref)
     check_lse(L, l_ref)
+    # the accumulator is only read
+    assert torch.equal(l_d.cpu(), l_in) and torch.equal(o_d.cpu().isnan(), o_in.isnan())
 
 
 def test_forward_kv_chunks_then_merge_equals_full_softmax(lvx):
