@@ -269,8 +269,11 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
             a.zero_()
             return a
 
+        # delta depends on O and dO alone, and all P blocks of both are here: one launch for
+        # all rows ahead of the rounds (a visit of a real ring would bring its own block's)
+        ops.bwd_preprocess(o_, do_, delta, 0, Lq)
+
         def one_round(r0, r1, acc, ws_r):
-            ops.bwd_preprocess(o_, do_, delta, r0, r1 - r0)
             ops.bwd(q_, k_, v_, do_, L_, delta, dq, acc[0].transpose(1, 2), acc[1].transpose(1, 2), sm_scale,
                     r0, r1 - r0, mask, accumulate_dkv=True, workspace=ws_r, bias=bias)
 
