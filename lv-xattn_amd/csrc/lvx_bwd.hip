@@ -441,13 +441,17 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         int rc = 0;       // i % 5
 
         auto step = [&](int i, bool s_live, bool pv_live, bool ds_live, bool copy) __attribute__((always_inline)) {
-            // A P-wave's part of tile i (requested two steps ago) must have landed.  When the
-            // previous step requested a tile, the wave has issued since: 2 dS^T stores,
-            // [wave 0: metadata loads,] 4 tile loads, 2 stores.  Loads complete in order, so
-            // "at most 4 operations outstanding" covers tile i and leaves tile i+1 in flight.
+            // A P-wave's part of tile i (requested two steps ago) must have landed.  Vector-memory
+            // operations complete in issue order, and after the loads of tile i the wave has issued
+            // at least: the 4 loads of tile i+1 (requested in step i-1, or in the prologue), and
+            // from step 5 on also the 2 dS^T stores of step i-2 and the 2 of step i-1 (steps 0-2
+            // store nothing; wave 0's metadata loads and the bias loads only add to this).  So "at
+            // most 8 outstanding" (4 in the first steps) says tile i is there and leaves everything
+            // younger in flight.
             if (!DROLE) {
-                if (i + 1 < n_iter) wait_vmcnt<4>();
-                else wait_vmcnt<0>();
+                if (i + 1 >= n_iter) wait_vmcnt<0>();
+                else if (i >= 5) wait_vmcnt<8>();
+                else wait_vmcnt<4>();
             }
             lds_barrier();
             // tile i+2 replaces tile i-3, whose last readers finished before this barrier
