@@ -68,6 +68,11 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     return bias
 
 
+def clear_mask_cache() -> None:
+    """Drops the converted mask `_mask_bias` keeps (an fp32 tensor of the mask's size)."""
+    _bias_cache.clear()
+
+
 def lv_xattn_attention_forward(module, query, key, value, attention_mask: Optional[torch.Tensor],
                                dropout: float = 0.0, scaling: Optional[float] = None, **kwargs):
     """Attention-interface function (same contract as transformers'
