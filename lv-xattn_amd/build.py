@@ -30,7 +30,7 @@ FLAGS = [
     # MFMA results in arch VGPRs (the VALU reads them without copies); the
     # register allocator then parks long-lived MFMA operands in AGPRs instead
     "-mllvm", "-amdgpu-mfma-vgpr-form",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
 
 
@@ -53,10 +53,27 @@ def _run(cmd, verbose):
         print(err)
 
 
+# hand-scheduled inner loops: (generator, arguments, include file it writes)
+GENERATED = [("gen_fwd_loop.py", ["bf16"], "lvx_fwd_loop_bf16.inc")]
+
+
+def generate() -> None:
+    """Runs the loop generators; an include file is rewritten only when its text changes."""
+    for gen, args, out in GENERATED:
+        r = subprocess.run([sys.executable, os.path.join(CSRC, gen), *args], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"{gen} failed:\n{r.stdout}\n{r.stderr}")
+        path = os.path.join(CSRC, out)
+        if not os.path.exists(path) or open(path).read() != r.stdout:
+            with open(path, "w") as f:
+                f.write(r.stdout)
+
+
 def build(force: bool = True, verbose: bool = False, extra_flags=()) -> str:
     os.makedirs(BUILD_DIR, exist_ok=True)
     cc = hipcc()
-    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    generate()
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".inc"))]
     headers.append(os.path.join(HERE, "..", "include", "lvx.h"))
     newest_hdr = max(os.path.getmtime(h) for h in headers)
     objs, jobs = [], []

@@ -323,6 +323,340 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     }
 }
 
+// registers the hand-scheduled loop uses besides its operands (see gen_fwd_loop.py)
+#define LVX_FWD_LOOP_CLOBBERS "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253"
+
+// The bf16 kernel without a dense bias (the one the benchmarks run): fwd_kernel's mapping, LDS
+// layout and tile code, but the run of key tiles that every row of the work-group sees in full
+// goes through a hand-scheduled loop (gen_fwd_loop.py) in which every wave interleaves the
+// MFMAs of a tile with the exponentials of that tile and the scores of the next one.  The
+// tiles before and after that run (mask edges, the partial last tile) take the plain tile code.
+template <bool MASKED>
+__global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
+    constexpr bool BIAS = false, F16 = false;
+    using E = Elt<F16>;
+    __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
+    __shared__ int red[4][4];
+
+    const int wid = xcd_remap(blockIdx.x, p.total_wg);
+    if (wid >= p.total_wg) return;
+    const int tile = wid % p.n_row_tiles;
+    const int t1 = wid / p.n_row_tiles;
+    const int split = t1 % p.nsplit;
+    const int t2 = t1 / p.nsplit;
+    // samples vary faster than head groups: every XCD (a contiguous range of ids) then gets
+    // work-groups of all samples, and ragged samples do not leave some XCDs idle early
+    const int b = t2 % p.B;
+    const int hg = t2 / p.B;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int h = hg * p.HG + (wave % p.HG);
+    const int hk = h / p.G;
+    const int row = p.row_begin + (tile * p.RS + wave / p.HG) * 32 + l32;
+    const bool row_ok = row < p.row_end;
+
+    int kv_len = p.Lkv;
+    if (p.kv_len) kv_len = min(p.kv_len[b], p.Lkv);
+    const int kv_lo = split * p.split_len;
+    const int kv_hi = min(kv_len, kv_lo + p.split_len);
+
+    // this lane's visible key interval
+    int my_s = kv_lo, my_e = kv_hi;
+    if (MASKED) {
+        if (row_ok) {
+            my_s = max(kv_lo, p.kv_start[(int64_t)b * p.Lq + row]);
+            my_e = min(kv_hi, p.kv_end[(int64_t)b * p.Lq + row]);
+        } else {
+            my_e = my_s;
+        }
+    }
+    if (my_e <= my_s) { my_s = BIG; my_e = 0; }
+
+    // work-group key range: [lo, hi) covers every non-empty row; tiles inside
+    // [in_lo, in_hi) are visible to every row and need no masking
+    int lo = my_s, hi = my_e, in_lo = my_s, in_hi = my_e;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        lo = min(lo, __shfl_xor(lo, off));
+        hi = max(hi, __shfl_xor(hi, off));
+        in_lo = max(in_lo, __shfl_xor(in_lo, off));
+        in_hi = min(in_hi, __shfl_xor(in_hi, off));
+    }
+    if (lane == 0) { red[wave][0] = lo; red[wave][1] = hi; red[wave][2] = in_lo; red[wave][3] = in_hi; }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        lo = min(lo, red[w][0]);
+        hi = max(hi, red[w][1]);
+        in_lo = max(in_lo, red[w][2]);
+        in_hi = min(in_hi, red[w][3]);
+    }
+    // the same in every lane of the work-group: keep them in scalar registers
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    in_lo = __builtin_amdgcn_readfirstlane(in_lo);
+    in_hi = __builtin_amdgcn_readfirstlane(in_hi);
+
+    // Q^T as B operand, resident for the whole kernel
+    bf16x8 qreg[8];
+    {
+        const uint16_t* qp = p.q + b * p.qs.b + h * p.qs.h + (int64_t)row * p.qs.s + g * 8;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) qreg[kk] = as_bf16x8(ldg16(qp + kk * 16, row_ok));
+    }
+
+    const char* kbase = reinterpret_cast<const char*>(p.k + b * p.ks.b + hk * p.ks.h);
+    const char* vbase = reinterpret_cast<const char*>(p.v + b * p.vs.b + hk * p.vs.h);
+    const uint32_t krow_b = (uint32_t)p.ks.s * 2u, vrow_b = (uint32_t)p.vs.s * 2u;   // bytes per key row
+
+    // global -> LDS: wave w moves the 1 KiB chunks w, w+4, w+8, w+12 (4 rows each)
+    // of the K tile and of the V tile; lane i fills position i & 15 of row i >> 4.
+    const int wave_u = wave;
+    const int ld_r = lane >> 4;
+    const uint32_t ld_c = (uint32_t)((lane & 15) ^ ((ld_r << 2) | wave_u)) * 16u;   // chunk this lane fetches
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&kv_lds[0][0][0];
+    auto issue = [&](int kv0, int buf) {
+        const char* kb = kbase + (int64_t)kv0 * krow_b;
+        const char* vb = vbase + (int64_t)kv0 * vrow_b;
+        const uint32_t slot = lds0 + (uint32_t)buf * (2 * TILE_BYTES) + (uint32_t)wave_u * 1024u;
+        const int last = kv_hi - 1 - kv0;          // rows past `last` repeat it
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = (uint32_t)min(4 * (wave_u + 4 * j) + ld_r, last);
+            dma16(kb, r * krow_b + ld_c, slot + j * 4096);
+            dma16(vb, r * vrow_b + ld_c, slot + TILE_BYTES + j * 4096);
+        }
+    };
+
+    // LDS -> operands.  K rows (A of S^T): 16 bytes at row * 256 + ((2 kk + g) ^ f(row)) * 16.
+    const int f_row = ((l32 & 3) << 2) | ((l32 >> 2) & 3);
+    const uint32_t k_rd = (uint32_t)(l32 * 256), k_h = (uint32_t)((g ^ f_row) << 4);
+    // V^T (A of O^T += V^T P^T), keys in accumulator order: first half rows 16 j + 4 g + r,
+    // second half 8 rows further down, whose f differs in bit 1.
+    uint32_t v_rd[4][2];
+    {
+        const int r = (lane & 15) >> 2, t = lane & 3, u = (lane >> 4) & 1;
+        const int low = (2 * u + (t >> 1)) ^ g;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            v_rd[dt][0] = (uint32_t)((4 * g + r) * 256 + (4 * (dt ^ r) + low) * 16 + (t & 1) * 8);
+            v_rd[dt][1] = (uint32_t)((4 * g + r + 8) * 256 + (4 * (dt ^ r) + (low ^ 2)) * 16 + (t & 1) * 8);
+        }
+    }
+
+    f32x16 acc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;
+    const float c = p.scale_log2e;
+    const float cc = BIAS ? 1.f : c;              // factor from the carried scores to log2 units
+    const float* brow = nullptr;                  // this lane's row of the bias
+    if (BIAS) brow = p.bias + b * p.bias_b + h * p.bias_h + (int64_t)min(row, p.row_end - 1) * p.bias_r;
+
+    const int t_begin = (hi > lo) ? lo / BN : 0;
+    const int t_end = (hi > lo) ? (hi + BN - 1) / BN : 0;
+
+    // the run [ta, ta + n_fast) of full tiles no row masks: an odd number of at least three
+    int ta = t_begin, n_fast = 0;
+    if (krow_b == vrow_b) {
+        const int fa = max(t_begin, (in_lo + BN - 1) / BN);
+        const int fb = min(t_end, min(in_hi, kv_hi) / BN);
+        if (fb - fa >= 3) { ta = fa; n_fast = (fb - fa - 1) | 1; }
+    }
+
+    for (int phase = 0; phase < 3; ++phase) {
+        if (phase == 1) {
+            if (n_fast == 0) continue;
+            int trips = n_fast >> 1;
+            const char* kp = kbase + (int64_t)(ta * BN) * krow_b;
+            const char* vp = vbase + (int64_t)(ta * BN) * vrow_b;
+            uint32_t doff[4], kaddr[8], vaddr[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) doff[j] = (uint32_t)(4 * (wave_u + 4 * j) + ld_r) * krow_b + ld_c;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) kaddr[kk] = lds0 + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) {
+                vaddr[2 * dt] = lds0 + TILE_BYTES + v_rd[dt][0];
+                vaddr[2 * dt + 1] = lds0 + TILE_BYTES + v_rd[dt][1];
+            }
+            const uint32_t lds_w = lds0 + (uint32_t)wave_u * 1024u;
+            asm volatile(
+#include "lvx_fwd_loop_bf16.inc"
+                : "+{v[0:15]}"(acc[0]), "+{v[16:31]}"(acc[1]), "+{v[32:47]}"(acc[2]), "+{v[48:63]}"(acc[3]),
+                  "+{v244}"(m_i), "+{v245}"(l_i), "+{s[44:45]}"(kp), "+{s[46:47]}"(vp), "+{s51}"(trips)
+                : "{v[64:67]}"(qreg[0]), "{v[68:71]}"(qreg[1]), "{v[72:75]}"(qreg[2]), "{v[76:79]}"(qreg[3]),
+                  "{v[80:83]}"(qreg[4]), "{v[84:87]}"(qreg[5]), "{v[88:91]}"(qreg[6]), "{v[92:95]}"(qreg[7]),
+                  "{v224}"(kaddr[0]), "{v225}"(kaddr[1]), "{v226}"(kaddr[2]), "{v227}"(kaddr[3]),
+                  "{v228}"(kaddr[4]), "{v229}"(kaddr[5]), "{v230}"(kaddr[6]), "{v231}"(kaddr[7]),
+                  "{v232}"(vaddr[0]), "{v233}"(vaddr[1]), "{v234}"(vaddr[2]), "{v235}"(vaddr[3]),
+                  "{v236}"(vaddr[4]), "{v237}"(vaddr[5]), "{v238}"(vaddr[6]), "{v239}"(vaddr[7]),
+                  "{v240}"(doff[0]), "{v241}"(doff[1]), "{v242}"(doff[2]), "{v243}"(doff[3]),
+                  "{s40}"(cc), "{s41}"(-INFINITY), "{s42}"(RESCALE_LOG2), "{s48}"((uint32_t)BN * krow_b),
+                  "{s49}"((uint32_t)BN * vrow_b), "{s50}"(lds_w)
+                : "memory", "vcc", "scc", "m0", "s52", "s53", "s54", "s55", "s56", LVX_FWD_LOOP_CLOBBERS);
+            continue;
+        }
+        const int t0 = phase == 0 ? t_begin : ta + n_fast;
+        const int t1 = phase == 0 ? ta : t_end;
+        if (t1 <= t0) continue;
+        __syncthreads();     // the tile buffers are free: every wave is done with the previous phase
+        issue(t0 * BN, 0);
+        for (int t = t0; t < t1; ++t) {
+            const int kv0 = t * BN;
+            const int buf = (t - t0) & 1;
+            const char* Ks = kv_lds[buf][0];
+            const char* Vs = kv_lds[buf][1];
+
+            // tile t has landed (this wave's part: vmcnt; everyone's: barrier); the
+            // barrier also says every wave is done reading tile t-1, whose buffer
+            // the loads of tile t+1 may now overwrite
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (t + 1 < t1) issue(kv0 + BN, buf ^ 1);
+
+            // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows.
+            // All 16 K operands are requested before the first MFMA, so the LDS
+            // latency is paid once per tile and not once per k-step.
+            bf16x8 ka[8][2];
+    #pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+                ka[kk][0] = *reinterpret_cast<const bf16x8*>(kp);
+                ka[kk][1] = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 s0, s1;
+    #pragma unroll
+            for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
+    #pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                s0 = E::mfma(ka[kk][0], qreg[kk], s0);
+                s1 = E::mfma(ka[kk][1], qreg[kk], s1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // V^T operands of this tile: requested now, they land during the softmax
+            u32x2 va[4][4][2];
+    #pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+    #pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    va[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
+                    va[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][1] + j * 4096));
+                }
+            __builtin_amdgcn_sched_barrier(0);
+
+            if (BIAS) {
+                // register group vg of lane-half g holds keys kv0 + 8 vg + 4 g + 0..3 (+32 for s1);
+                // groups past the end re-read the last one (those keys are masked below)
+    #pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int k0 = kv0 + 8 * vg + 4 * g;
+                    const f32x4 ba = *reinterpret_cast<const f32x4*>(brow + min(k0, (p.Lkv - 1) & ~3));
+                    const f32x4 bb = *reinterpret_cast<const f32x4*>(brow + min(k0 + 32, (p.Lkv - 1) & ~3));
+    #pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        s0[4 * vg + r] = fmaf(s0[4 * vg + r], c, ba[r] * LOG2E_F);
+                        s1[4 * vg + r] = fmaf(s1[4 * vg + r], c, bb[r] * LOG2E_F);
+                    }
+                }
+            }
+
+            if (kv0 < in_lo || kv0 + BN > in_hi) {
+    #pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int kv = kv0 + acc_row(v, g);
+                    if (kv < my_s || kv >= my_e) s0[v] = -INFINITY;
+                    if (kv + 32 < my_s || kv + 32 >= my_e) s1[v] = -INFINITY;
+                }
+            }
+
+            float mx = max3(s0[0], s1[0], s0[1]);
+            mx = max3(mx, s1[1], s0[2]);
+    #pragma unroll
+            for (int v = 3; v < 16; v += 1) mx = max3(mx, s1[v - 1], s0[v]);
+            mx = fmaxf(mx, s1[15]);
+            {   // other half of the wave holds the other 32 keys of the same text row
+                const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+                mx = max3(__uint_as_float(sw[0]), __uint_as_float(sw[1]), m_i);
+            }
+            // Lazy rescale: the reference point m_i of a row only moves when the row
+            // maximum has grown by more than 2^RESCALE_LOG2 since it was set, so P may
+            // reach 2^RESCALE_LOG2 instead of 1 (harmless in fp32 / bf16) and the
+            // rescale of O happens a few times per row instead of almost every tile.
+            const float mcand = mx * cc;                      // mx >= m_i
+            const float m_ic = m_i * cc;
+            const bool move = (mx != -INFINITY) && !(mcand - m_ic <= RESCALE_LOG2);
+            const float alpha = move ? __builtin_amdgcn_exp2f(m_ic - mcand) : 1.f;
+            if (move) m_i = mx;
+            const float mc = (m_i == -INFINITY) ? 0.f : m_i * cc;
+
+            // P^T as B operand: k-step j covers keys 16j..16j+15 of the tile.  The row
+            // sum is taken in fp32 before the rounding to bf16 (summing the rounded
+            // values would put the LSE off by up to a bf16 ulp of the largest term).
+            bf16x8 pb[4];
+            float rs0 = 0.f, rs1 = 0.f;
+    #pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                u32x4 u0, u1;
+    #pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 8 * j + 2 * e;
+                    const float a0 = __builtin_amdgcn_exp2f(fmaf(s0[v], cc, -mc)), a1 = __builtin_amdgcn_exp2f(fmaf(s0[v + 1], cc, -mc));
+                    const float b0 = __builtin_amdgcn_exp2f(fmaf(s1[v], cc, -mc)), b1 = __builtin_amdgcn_exp2f(fmaf(s1[v + 1], cc, -mc));
+                    rs0 += a0 + a1;
+                    rs1 += b0 + b1;
+                    u0[e] = E::pack(a0, a1);
+                    u1[e] = E::pack(b0, b1);
+                }
+                pb[j] = as_bf16x8(u0);
+                pb[2 + j] = as_bf16x8(u1);
+            }
+            l_i = l_i * alpha + (rs0 + rs1);
+
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {   // the running max moved for some row
+    #pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+    #pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[dt][v] *= alpha;
+            }
+
+            // O^T += V^T P^T
+            __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+    #pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const u32x4 a = {va[dt][j][0][0], va[dt][j][0][1], va[dt][j][1][0], va[dt][j][1][1]};
+                    acc[dt] = E::mfma(as_bf16x8(a), pb[j], acc[dt]);
+                }
+        }
+    }
+
+    // epilogue: the two lane halves hold partial row sums of the same row
+    const float l_tot = l_i + __shfl_xor(l_i, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (row_ok) {
+        uint16_t* op = p.o + split * p.o_split_stride + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int vg = 0; vg < 4; ++vg) {
+                u32x2 w;
+                w[0] = E::pack(acc[dt][4 * vg] * inv, acc[dt][4 * vg + 1] * inv);
+                w[1] = E::pack(acc[dt][4 * vg + 2] * inv, acc[dt][4 * vg + 3] * inv);
+                *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * vg + 4 * g) = w;
+            }
+        if (g == 0) {
+            const float lse = l_tot > 0.f ? m_i * (BIAS ? LN2_F : p.scale) + __logf(l_tot) : -INFINITY;
+            p.lse[split * p.lse_split_stride + ((int64_t)b * p.Hq + h) * p.lse_bh_stride + row] = lse;
+        }
+    }
+}
+
 }  // namespace
 
 namespace {
@@ -332,6 +666,9 @@ hipError_t launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
     if (p.bias) {
         if (masked) return launch1((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), st, p);
         else return launch1((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), st, p);
+    } else if (!F16) {
+        if (masked) return launch1((fwd_kernel_pipe<true>), dim3(grid), dim3(256), st, p);
+        else return launch1((fwd_kernel_pipe<false>), dim3(grid), dim3(256), st, p);
     } else {
         if (masked) return launch1((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), st, p);
         else return launch1((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), st, p);
