@@ -54,7 +54,9 @@ def _run(cmd, verbose):
 
 
 # hand-scheduled inner loops: (generator, arguments, include file it writes)
-GENERATED = [("gen_fwd_loop.py", ["bf16"], "lvx_fwd_loop_bf16.inc")]
+GENERATED = [("gen_fwd_loop.py", ["bf16"], "lvx_fwd_loop_bf16.inc"),
+             ("gen_bwd_loop.py", ["p"], "lvx_bwd_loop_p.inc"),
+             ("gen_bwd_loop.py", ["d"], "lvx_bwd_loop_d.inc")]
 
 
 def generate() -> None:

@@ -27,7 +27,7 @@
 //
 // All MFMA are 32x32x16 bf16.  A operands come from LDS.  The Q and dO tiles
 // ([32 rows][128] bf16, 8 KiB each) go from global memory straight into LDS
-// with global_load_lds_dwordx4, two steps ahead, into a ring of five buffers;
+// with global_load_lds_dwordx4, two steps ahead, into rings of six buffers;
 // the load writes 64 lanes x 16 bytes contiguously, so rows are not padded:
 // the 16-byte chunk c of row r is kept at position c ^ f(r),
 // f(r) = ((r & 3) << 2) | ((r >> 2) & 3), which makes both access patterns
@@ -51,14 +51,16 @@ constexpr int BM = 32;        // text rows per step
 constexpr int NT = 512;       // threads per work-group
 constexpr int DSS = BM + 8;   // row stride of the dS^T tile [token][row]
 
-// LDS map (uint16 units): a ring of five (Q | dO) tile pairs, unpadded; two dS^T tiles; two P hand-over buffers
+// LDS map (uint16 units): a ring of six Q tiles, a ring of six dO tiles (each ring within the 64 KiB an LDS
+// instruction's immediate offset reaches from one address register), unpadded; two dS^T tiles; two P
+// hand-over buffers
 constexpr int TILE_ELEMS = BM * D;             // one Q or dO tile (8 KiB)
-constexpr int QD_ELEMS = 2 * TILE_ELEMS;
-constexpr int NQD = 5;
+constexpr int NQD = 6;
 constexpr int DST_ELEMS = BN * DSS;
 constexpr int PB_ELEMS = 4 * 2 * 64 * 8;       // P hand-over: [slice][half][lane][16 bytes] as uint16
-constexpr int OFF_QD = 0;                      // x NQD
-constexpr int OFF_DST = OFF_QD + NQD * QD_ELEMS; // x2
+constexpr int OFF_Q = 0;                       // x NQD
+constexpr int OFF_DO = OFF_Q + NQD * TILE_ELEMS; // x NQD
+constexpr int OFF_DST = OFF_DO + NQD * TILE_ELEMS; // x2
 constexpr int OFF_PB = OFF_DST + 2 * DST_ELEMS;  // x2
 constexpr int LOOP_ELEMS = OFF_PB + 2 * PB_ELEMS;
 constexpr int EPS = D + 1;                          // row stride (floats) of the epilogue's transposed tile
@@ -66,6 +68,9 @@ constexpr int EPI_ELEMS = 8 * 32 * EPS * 2;         // 8 waves x [32 tokens][128
 constexpr int SMEM_ELEMS = LOOP_ELEMS > EPI_ELEMS ? LOOP_ELEMS : EPI_ELEMS;
 
 constexpr float LOG2E = 1.4426950408889634f;
+
+// registers the hand-scheduled loops use besides their operands (see gen_bwd_loop.py)
+#define LVX_BWD_LOOP_CLOBBERS "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199"
 
 // BIAS: a dense fp32 bias joins the exponent, P = exp2(S*c + bias*log2e - LSE*log2e).
 template <bool MASKED, bool BIAS, bool F16>
@@ -210,11 +215,11 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
         const uint32_t row0 = (uint32_t)min(r0 + ld_r, p.row_end - 1);
         const uint32_t row1 = (uint32_t)min(r0 + ld_r + 4, p.row_end - 1);
-        const uint32_t slot = lds0 + (uint32_t)buf * (QD_ELEMS * 2) + (uint32_t)slice * 2048u;
+        const uint32_t slot = lds0 + (uint32_t)buf * (TILE_ELEMS * 2) + (uint32_t)slice * 2048u;
         dma16(q_head, row0 * qrow_b + ld_c0, slot);
         dma16(q_head, row1 * qrow_b + ld_c1, slot + 1024);
-        dma16(do_head, row0 * dorow_b + ld_c0, slot + TILE_ELEMS * 2);
-        dma16(do_head, row1 * dorow_b + ld_c1, slot + TILE_ELEMS * 2 + 1024);
+        dma16(do_head, row0 * dorow_b + ld_c0, slot + OFF_DO * 2);
+        dma16(do_head, row1 * dorow_b + ld_c1, slot + OFF_DO * 2 + 1024);
     };
     auto advance = [&]() {   // next (head, row tile) of the walk, wrapping
         ++cur_qt;
@@ -257,8 +262,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) bv[v] = bp[(int64_t)min(8 * (v >> 2) + 4 * g + (v & 3), last) * p.bias_r];
         }
-        const char* qt = reinterpret_cast<const char*>(tile_cur);
-        const char* dot = reinterpret_cast<const char*>(tile_prev) + TILE_ELEMS * 2;
+        const char* qt = reinterpret_cast<const char*>(tile_cur);     // Q of tile i
+        const char* dot = reinterpret_cast<const char*>(tile_prev);   // dO of tile i-1
         bf16x8 qa[8];
         u32x2 da[4][2][2];
         // MASKED: lane l looks at the key interval of row l of the previous tile (requested
@@ -342,7 +347,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 
     auto d_step = [&](bool pv_live, bool ds_live, const uint16_t* tile_p1, const uint16_t* tile_p2, const u32x4* meta,
                       const uint16_t* pbuf, uint16_t* dst, f32x16& dp_carry) __attribute__((always_inline)) {
-        const char* dor = reinterpret_cast<const char*>(tile_p1) + TILE_ELEMS * 2;   // dO rows of tile i-1
+        const char* dor = reinterpret_cast<const char*>(tile_p1);                    // dO rows of tile i-1
         const char* qt = reinterpret_cast<const char*>(tile_p2);                     // Q of tile i-2
         u32x4 pu[2];
         u32x2 qa[4][2][2];
@@ -409,11 +414,12 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     auto run = [&](auto tail_c, auto role_c) {
         constexpr bool DROLE = decltype(role_c)::value;
         if (n_iter == 0) return;
-        // tile i lives in qd(i % 5) with its row metadata in meta_s4[i % 5]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
-        auto qd = [&](int k) { return smem + OFF_QD + k * QD_ELEMS; };
+        // tile i lives in qt(i % 6) / dot(i % 6) with its row metadata in meta_s4[i % 6]; P(i) in pbf(i & 1); dS^T(i) in dst(i & 1)
+        auto qt = [&](int k) { return smem + OFF_Q + k * TILE_ELEMS; };
+        auto dot = [&](int k) { return smem + OFF_DO + k * TILE_ELEMS; };
         auto dst = [&](int k) { return smem + OFF_DST + k * DST_ELEMS; };
         auto pbf = [&](int k) { return smem + OFF_PB + k * PB_ELEMS; };
-        auto m5 = [](int x) { return x >= NQD ? x - NQD : x; };
+        auto m6 = [](int x) { return x >= NQD ? x - NQD : x; };
         // dS^T workspace offsets of the tiles in flight: a tile enters at [5] when requested
         // (two steps ahead); at step i (before that step's shift) tile i is at [3], tile i-3 at [0]
         int64_t w_q[6] = {0, 0, 0, 0, 0, 0};
@@ -438,7 +444,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         f32x16 carry;     // P-wave: raw S of the previous tile; D-wave: dP of the previous tile
 #pragma unroll
         for (int v = 0; v < 16; ++v) carry[v] = 0.f;
-        int rc = 0;       // i % 5
+        int rc = 0;       // i % 6
 
         auto step = [&](int i, bool s_live, bool pv_live, bool ds_live, bool copy) __attribute__((always_inline)) {
             // A P-wave's part of tile i (requested two steps ago) must have landed.  Vector-memory
@@ -454,18 +460,18 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 else wait_vmcnt<4>();
             }
             lds_barrier();
-            // tile i+2 replaces tile i-3, whose last readers finished before this barrier
-            if (i + 2 < n_iter) fetch(m5(rc + 2));
-            const int r1 = m5(rc + 4), r2 = m5(rc + 3);     // (i - 1) % 5, (i - 2) % 5
+            // tile i+2 replaces tile i-4, whose last readers finished long before this barrier
+            if (i + 2 < n_iter) fetch(m6(rc + 2));
+            const int r1 = m6(rc + 5), r2 = m6(rc + 4);     // (i - 1) % 6, (i - 2) % 6
             if (!DROLE)
-                p_step(tail_c, s_live, pv_live, qd(rc), qd(r1), meta_s4[r1], pbf((i + 1) & 1), carry, b_q[2], r_q[2]);
+                p_step(tail_c, s_live, pv_live, qt(rc), dot(r1), meta_s4[r1], pbf((i + 1) & 1), carry, b_q[2], r_q[2]);
             else
-                d_step(pv_live, ds_live, qd(r1), qd(r2), meta_s4[r2], pbf(i & 1), dst(i & 1), carry);
+                d_step(pv_live, ds_live, dot(r1), qt(r2), meta_s4[r2], pbf(i & 1), dst(i & 1), carry);
             // dS^T(i-3) to HBM last: its LDS read queues behind this step's operand reads
             // instead of delaying them, and only has to finish before the next barrier
             if (!DROLE && copy) copy_out(dst((i + 1) & 1), w_q[0]);
             shift();
-            rc = m5(rc + 1);
+            rc = m6(rc + 1);
         };
         fetch(0);
         shift();
@@ -474,6 +480,95 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         const int last = n_iter + 1;
         int i = 0;
         for (; i < 3 && i <= last; ++i) step(i, i < n_iter, i >= 1 && i <= n_iter, i >= 2, false);
+        // Steady state of the plain bf16 kernel: steps 3 .. 3 + 6 trips - 1 (every one of them with all
+        // its parts alive and a tile to request) run in the hand-scheduled loops of gen_bwd_loop.py,
+        // six steps a trip; the steps after them continue below as if they had run here.
+        if constexpr (!MASKED && !BIAS && !F16 && !decltype(tail_c)::value) {
+            int trips = uniform32((n_iter - 5) / 6);
+            if (i == 3 && trips >= 1 && (p.row_end - p.row_begin) % BM == 0) {
+                const int steps = 6 * trips;
+                uint32_t ra[8], ta[8];
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk)
+                    ra[kk] = lds0 + (DROLE ? OFF_DO : OFF_Q) * 2 + row_rd + ((uint32_t)(kk * 32) ^ row_h);
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt) {
+                    ta[2 * dt] = lds0 + (DROLE ? OFF_Q : OFF_DO) * 2 + t_rd[dt][0];
+                    ta[2 * dt + 1] = lds0 + (DROLE ? OFF_Q : OFF_DO) * 2 + t_rd[dt][1];
+                }
+                const uint32_t a_pb = lds0 + OFF_PB * 2 + (uint32_t)pb_off * 2;
+                const uint32_t a_meta = meta0 + (uint32_t)g * 16u;
+                if constexpr (!DROLE) {
+                    uint16_t* ws_k = p.ds_ws + (int64_t)kblk * p.ws_ld;
+                    const char* qp = uniform_ptr(q_head + (int64_t)(p.row_begin + cur_qt * BM) * qrow_b);
+                    const char* dop = uniform_ptr(do_head + (int64_t)(p.row_begin + cur_qt * BM) * dorow_b);
+                    const char* mp = uniform_ptr(reinterpret_cast<const char*>(meta_head + cur_qt * 64));
+                    const char* wn = uniform_ptr(reinterpret_cast<const char*>(ws_k + ws_head + (int64_t)cur_qt * (BN * BM)));
+                    const char* w0 = uniform_ptr(reinterpret_cast<const char*>(ws_k + w_q[0]));
+                    const char* w1 = uniform_ptr(reinterpret_cast<const char*>(ws_k + w_q[1]));
+                    const char* w2 = uniform_ptr(reinterpret_cast<const char*>(ws_k + w_q[2]));
+                    const char* w3 = uniform_ptr(reinterpret_cast<const char*>(ws_k + w_q[3]));
+                    const char* w4 = uniform_ptr(reinterpret_cast<const char*>(ws_k + w_q[4]));
+                    const char* w5 = w4;
+                    int left = uniform32(cur_left);
+                    const int64_t hdq = uniform64((int64_t)p.qs.h * 2 - (int64_t)n_qtiles * BM * qrow_b);
+                    const int64_t hddo = uniform64((int64_t)p.dos.h * 2 - (int64_t)n_qtiles * BM * dorow_b);
+                    const int64_t hdws = uniform64((int64_t)p.ws_bh * 2 - (int64_t)n_qtiles * (BN * BM * 2));
+                    const uint32_t a_cp = lds0 + OFF_DST * 2 + (uint32_t)(cp_token * DSS + cp_part * 8) * 2;
+                    const uint32_t g_cp0 = (uint32_t)(cp_token * BM + cp_part * 8) * 2, g_cp1 = g_cp0 + 64 * BM * 2;
+                    const uint32_t lr = (uint32_t)(lane >> 4) + 8u * slice;
+                    const uint32_t g_q0 = lr * qrow_b + ld_c0, g_q1 = (lr + 4) * qrow_b + ld_c1;
+                    const uint32_t g_d0 = lr * dorow_b + ld_c0, g_d1 = (lr + 4) * dorow_b + ld_c1;
+                    wait_vmcnt<4>();    // tile 3 (the loads of tile 4 may be in flight); the loop counts from there
+                    asm volatile(
+#include "lvx_bwd_loop_p.inc"
+                        : "+{v[0:15]}"(acc[0]), "+{v[16:31]}"(acc[1]), "+{v[32:47]}"(acc[2]), "+{v[48:63]}"(acc[3]),
+                          "+{v[96:111]}"(carry), "+{s[44:45]}"(qp), "+{s[46:47]}"(dop), "+{s[48:49]}"(mp), "+{s[50:51]}"(wn),
+                          "+{s52}"(left), "+{s64}"(trips), "+{s[66:67]}"(w0), "+{s[68:69]}"(w1), "+{s[70:71]}"(w2),
+                          "+{s[72:73]}"(w3), "+{s[74:75]}"(w4), "+{s[76:77]}"(w5)
+                        : "{v[64:67]}"(breg[0]), "{v[68:71]}"(breg[1]), "{v[72:75]}"(breg[2]), "{v[76:79]}"(breg[3]),
+                          "{v[80:83]}"(breg[4]), "{v[84:87]}"(breg[5]), "{v[88:91]}"(breg[6]), "{v[92:95]}"(breg[7]),
+                          "{v200}"(ra[0]), "{v201}"(ra[1]), "{v202}"(ra[2]), "{v203}"(ra[3]),
+                          "{v204}"(ra[4]), "{v205}"(ra[5]), "{v206}"(ra[6]), "{v207}"(ra[7]),
+                          "{v208}"(ta[0]), "{v209}"(ta[1]), "{v210}"(ta[2]), "{v211}"(ta[3]),
+                          "{v212}"(ta[4]), "{v213}"(ta[5]), "{v214}"(ta[6]), "{v215}"(ta[7]),
+                          "{v216}"(a_pb), "{v217}"(a_meta), "{v218}"(a_cp), "{v219}"(g_cp0), "{v220}"(g_cp1),
+                          "{v221}"(g_q0), "{v222}"(g_q1), "{v223}"(g_d0), "{v224}"(g_d1), "{v225}"((uint32_t)lane * 4u),
+                          "{s40}"(uniform32(c)), "{s41}"(uniform32((uint32_t)BM * qrow_b)), "{s42}"(uniform32((uint32_t)BM * dorow_b)), "{s53}"(uniform32(n_qtiles)),
+                          "{s[54:55]}"(hdq), "{s[56:57]}"(hddo), "{s[60:61]}"(hdws),
+                          "{s62}"(uniform32(lds0 + (uint32_t)slice * 2048u)), "{s63}"(uniform32(meta0)), "{s65}"(uniform32(wave == 0 ? 1 : 0))
+                        : "memory", "vcc", "scc", "m0", LVX_BWD_LOOP_CLOBBERS);
+                    wait_vmcnt<0>();    // the steps below count the operations in flight from scratch
+                    w_q[0] = reinterpret_cast<const uint16_t*>(w0) - ws_k;
+                    w_q[1] = reinterpret_cast<const uint16_t*>(w1) - ws_k;
+                    w_q[2] = reinterpret_cast<const uint16_t*>(w2) - ws_k;
+                    w_q[3] = reinterpret_cast<const uint16_t*>(w3) - ws_k;
+                    w_q[4] = reinterpret_cast<const uint16_t*>(w4) - ws_k;
+                } else {
+                    const uint32_t a_ds = lds0 + OFF_DST * 2 + (uint32_t)((32 * slice + l32) * DSS + 4 * g) * 2;
+                    asm volatile(
+#include "lvx_bwd_loop_d.inc"
+                        : "+{v[0:15]}"(acc[0]), "+{v[16:31]}"(acc[1]), "+{v[32:47]}"(acc[2]), "+{v[48:63]}"(acc[3]),
+                          "+{v[96:111]}"(carry), "+{s64}"(trips)
+                        : "{v[64:67]}"(breg[0]), "{v[68:71]}"(breg[1]), "{v[72:75]}"(breg[2]), "{v[76:79]}"(breg[3]),
+                          "{v[80:83]}"(breg[4]), "{v[84:87]}"(breg[5]), "{v[88:91]}"(breg[6]), "{v[92:95]}"(breg[7]),
+                          "{v200}"(ra[0]), "{v201}"(ra[1]), "{v202}"(ra[2]), "{v203}"(ra[3]),
+                          "{v204}"(ra[4]), "{v205}"(ra[5]), "{v206}"(ra[6]), "{v207}"(ra[7]),
+                          "{v208}"(ta[0]), "{v209}"(ta[1]), "{v210}"(ta[2]), "{v211}"(ta[3]),
+                          "{v212}"(ta[4]), "{v213}"(ta[5]), "{v214}"(ta[6]), "{v215}"(ta[7]),
+                          "{v216}"(a_pb), "{v217}"(a_meta), "{v218}"(a_ds), "{s40}"(uniform32(p.scale))
+                        : "memory", "vcc", "scc", LVX_BWD_LOOP_CLOBBERS, "v219", "v220", "v221", "v222");
+                }
+                i += steps;
+                // the walk stands at the tile after the last one requested
+                const int pos = it_lo + i + 2;
+                cur_gi = pos / n_live;
+                cur_qt = pos % n_live;
+                cur_left = n_live - cur_qt;
+                if (cur_gi >= p.G) cur_gi = 0;
+                enter_head();
+            }
+        }
         for (; i < n_iter; ++i) step(i, true, true, true, true);
         for (; i <= last; ++i) step(i, false, i <= n_iter, true, true);
         __syncthreads();

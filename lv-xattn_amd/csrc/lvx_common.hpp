@@ -157,6 +157,18 @@ __device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)"
 // waited for separately, stores - are not waited for, as __syncthreads() would.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Values that are the same in every lane, made so for the compiler too (an inline-asm operand in a
+// scalar register must not look lane-dependent).
+__device__ __forceinline__ uint32_t uniform32(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ int uniform32(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ float uniform32(float x) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x))); }
+__device__ __forceinline__ int64_t uniform64(int64_t x) {
+    const uint32_t lo = uniform32((uint32_t)x), hi = uniform32((uint32_t)((uint64_t)x >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* x) { return reinterpret_cast<const T*>(uniform64((int64_t)(uintptr_t)x)); }
+
 // max of three (one instruction; fmaxf chains cost an extra canonicalising
 // v_max per MFMA result)
 __device__ __forceinline__ float max3(float a, float b, float c) {

@@ -421,9 +421,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
         const char* vb = vbase + (int64_t)kv0 * vrow_b;
         const uint32_t slot = lds0 + (uint32_t)buf * (2 * TILE_BYTES) + (uint32_t)wave_u * 1024u;
         const int last = kv_hi - 1 - kv0;          // rows past `last` repeat it
+        int lr = ld_r + 4 * wave_u;                // (a fresh copy: see the tile loop)
+        asm volatile("" : "+v"(lr));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const uint32_t r = (uint32_t)min(4 * (wave_u + 4 * j) + ld_r, last);
+            const uint32_t r = (uint32_t)min(lr + 16 * j, last);
             dma16(kb, r * krow_b + ld_c, slot + j * 4096);
             dma16(vb, r * vrow_b + ld_c, slot + TILE_BYTES + j * 4096);
         }
@@ -445,6 +447,14 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
         }
     }
 
+    // The same addresses as absolute LDS byte addresses for buffer 0.  The swizzles only touch address
+    // bits that nothing else sets, so the address of k-step kk (K) or d tile dt (V) is the first one
+    // with kk * 32 or dt * 64 XORed in: three registers serve the plain tile code and the
+    // hand-scheduled loop (which wants all sixteen spelled out) alike.
+    const uint32_t kaddr0 = lds0 + k_rd + k_h;
+    const uint32_t vaddr0 = lds0 + TILE_BYTES + v_rd[0][0], vaddr1 = lds0 + TILE_BYTES + v_rd[0][1];
+    const char* const lds_base = &kv_lds[0][0][0] - lds0;     // LDS byte address -> pointer
+
     f32x16 acc[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -464,7 +474,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
     if (krow_b == vrow_b) {
         const int fa = max(t_begin, (in_lo + BN - 1) / BN);
         const int fb = min(t_end, min(in_hi, kv_hi) / BN);
+#ifndef LVX_FWD_NOFAST
         if (fb - fa >= 3) { ta = fa; n_fast = (fb - fa - 1) | 1; }
+#endif
     }
 
     for (int phase = 0; phase < 3; ++phase) {
@@ -477,11 +489,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) doff[j] = (uint32_t)(4 * (wave_u + 4 * j) + ld_r) * krow_b + ld_c;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) kaddr[kk] = lds0 + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+            for (int kk = 0; kk < 8; ++kk) kaddr[kk] = kaddr0 ^ (uint32_t)(kk * 32);
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
-                vaddr[2 * dt] = lds0 + TILE_BYTES + v_rd[dt][0];
-                vaddr[2 * dt + 1] = lds0 + TILE_BYTES + v_rd[dt][1];
+                vaddr[2 * dt] = vaddr0 ^ (uint32_t)(dt * 64);
+                vaddr[2 * dt + 1] = vaddr1 ^ (uint32_t)(dt * 64);
             }
             const uint32_t lds_w = lds0 + (uint32_t)wave_u * 1024u;
             asm volatile(
@@ -508,8 +520,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
         for (int t = t0; t < t1; ++t) {
             const int kv0 = t * BN;
             const int buf = (t - t0) & 1;
-            const char* Ks = kv_lds[buf][0];
-            const char* Vs = kv_lds[buf][1];
+            // fresh copies the compiler cannot hoist: the sixteen derived addresses are then formed
+            // tile by tile (an XOR each) instead of being kept - and spilled - across the whole loop
+            uint32_t ka0 = kaddr0, va0 = vaddr0, va1 = vaddr1;
+            asm volatile("" : "+v"(ka0), "+v"(va0), "+v"(va1));
 
             // tile t has landed (this wave's part: vmcnt; everyone's: barrier); the
             // barrier also says every wave is done reading tile t-1, whose buffer
@@ -524,7 +538,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
             bf16x8 ka[8][2];
     #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
-                const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
+                const char* kp = lds_base + (ka0 ^ (uint32_t)(kk * 32)) + buf * (2 * TILE_BYTES);
                 ka[kk][0] = *reinterpret_cast<const bf16x8*>(kp);
                 ka[kk][1] = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
             }
@@ -544,8 +558,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel_pipe(const FwdParams p) {
             for (int dt = 0; dt < 4; ++dt)
     #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    va[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
-                    va[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][1] + j * 4096));
+                    va[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(lds_base + (va0 ^ (uint32_t)(dt * 64)) + buf * (2 * TILE_BYTES) + j * 4096));
+                    va[dt][j][1] = lds_read_tr16(reinterpret_cast<const uint16_t*>(lds_base + (va1 ^ (uint32_t)(dt * 64)) + buf * (2 * TILE_BYTES) + j * 4096));
                 }
             __builtin_amdgcn_sched_barrier(0);
 

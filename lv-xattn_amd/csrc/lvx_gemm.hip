@@ -22,6 +22,8 @@
 //    is kept as it lies, [k][rows], and read with the transposing LDS read.
 //  * The MFMA computes C^T (A operand = rows of the B tile), so a lane ends up
 //    with 4 consecutive columns of one C row and stores 8 bytes.
+#include <type_traits>
+
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -108,6 +110,8 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     constexpr int LPG_A = RA::CHUNKS / 8;
     static_assert(RA::CHUNKS % 8 == 0 && RB::CHUNKS % 8 == 0, "chunks split evenly over 8 waves");
     constexpr int NRA = RA::NRD(WM), NRB = RB::NRD(WN);
+    // LDS read instructions per MFMA of a stage (a transposing operand read is two)
+    constexpr int LDS_PER_MFMA = (2 * (WM * (A_MCONTIG ? 2 : 1) + WN * (B_NCONTIG ? 2 : 1)) + 2 * WM * WN - 1) / (2 * WM * WN);
     __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
     const int wid0 = xcd_remap(blockIdx.x, p.total_wg);
@@ -210,6 +214,56 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
+#ifdef LVX_GEMM_PIPE
+    // Every wave software-pipelines by itself: the operands of stage s+1 are read from LDS into a second
+    // register set while the 16 MFMAs of stage s issue, one barrier per stage.
+    bf16x8 am[2][2][WM], bn[2][2][WN];      // [register set][k-step][tile]
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s)
+        if (s < steps) issue(s);
+    if (steps > NS - 2) wait_vmcnt<(NS - 2) * LPG>();
+    else wait_vmcnt<0>();
+    phase_barrier();
+    auto fetch = [&](auto set_c, int s) __attribute__((always_inline)) {
+        constexpr int RS = decltype(set_c)::value;
+        const uint32_t base = (uint32_t)(s % NS) * STAGE;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int t = 0; t < WM; ++t) am[RS][kk][t] = RA::operand(lds, base, rda, t, kk);
+#pragma unroll
+            for (int t = 0; t < WN; ++t) bn[RS][kk][t] = RB::operand(lds, base + RA::BYTES, rdb, t, kk);
+        }
+    };
+    auto stage = [&](auto set_c, int s) __attribute__((always_inline)) {
+        constexpr int RS = decltype(set_c)::value;
+        // stage s+1 has landed (this wave's chunks: vmcnt; everyone's: barrier); every wave has read stage s-1
+        if (s + NS - 2 < steps) wait_vmcnt<(NS - 3) * LPG>();
+        else wait_vmcnt<0>();
+        wait_lds();
+        __builtin_amdgcn_s_barrier();
+        if (s + NS - 1 < steps) issue(s + NS - 1);
+        if (s + 1 < steps) fetch(std::integral_constant<int, RS ^ 1>{}, s + 1);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = E::mfma(bn[RS][kk][nt], am[RS][kk][mt], acc[nt][mt]);
+        // spread the MFMAs over the LDS reads and the global loads
+#pragma unroll
+        for (int i = 0; i < 2 * WM * WN; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, LDS_PER_MFMA, 0);   // LDS reads
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a vector-memory read, while there are any
+        }
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    for (int s = 0; s < steps; s += 2) {
+        stage(std::integral_constant<int, 0>{}, s);
+        if (s + 1 < steps) stage(std::integral_constant<int, 1>{}, s + 1);
+    }
+#else
     // prologue: stages 0 .. NS-2 in flight, stage 0 landed
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s)
@@ -253,6 +307,8 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
         phase_barrier();
     }
     if (set == 0) phase_barrier();
+
+#endif
 
     // C^T tile: accumulator rows = n, cols = m
     if (nks > 1) {   // partial tile of a split contraction: fp32, into this split's slice
