@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define LVX_VERSION 100
+#define LVX_VERSION 101
 
 #define LVX_OK 0
 #define LVX_ERR_NULL (-1)        /* a required pointer is NULL */
@@ -101,8 +101,9 @@ int lvx_fwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* 
  * lvx_fwd whose result is merged with an incoming accumulator (o_in [like o], l_in
  * [B*Hq, Lq], only read) before it is written to (o, lse): one round's _fwd_kernel launch plus
  * its _rescale_kernel launch (lv_xattn/attn.py:390-400 and 403-419) in one call.  With key
- * splits the partials and the accumulator are folded by the same merge launch; o must not be
- * o_in (LVX_ERR_SHAPE).  Workspace as for lvx_fwd.
+ * splits the partials and the accumulator are folded by the same merge launch.  The kernel writes
+ * (o, lse) before the merge reads (o_in, l_in): o may not overlap o_in and lse may not overlap l_in
+ * over the rows of the window (LVX_ERR_SHAPE).  Workspace as for lvx_fwd.
  */
 int lvx_fwd_acc(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
                 const lvx_tensor* o_in, const float* l_in, const lvx_tensor* o, float* lse,

@@ -36,6 +36,9 @@ import sys
 # experiment switches (comma separated in LVX_GEN_OPTS); none is set in a normal build
 OPTS = dict((o.split("=") + ["1"])[:2] for o in os.environ.get("LVX_GEN_OPTS", "").split(",") if o)
 ROLE = sys.argv[1] if len(sys.argv) > 1 else "p"
+for _o in list(OPTS):      # a switch for one role only: p_novalu, d_nolds, ...
+    if _o.startswith(ROLE + "_"):
+        OPTS[_o[2:]] = OPTS[_o]
 F16 = False
 MFMA = "v_mfma_f32_32x32x16_bf16"
 

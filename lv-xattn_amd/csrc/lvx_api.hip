@@ -242,7 +242,26 @@ int lvx_fwd_acc(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* 
     if (!o_in) return LVX_ERR_NULL;
     LVX_TRY(check_tensor(o_in));
     if (!l_in) return LVX_ERR_NULL;
-    if (o && o_in->ptr == o->ptr) return LVX_ERR_SHAPE;     // the result is formed out of place
+    // the result is formed out of place: the kernel writes (o, lse) of the window before the merge
+    // reads (o_in, l_in), so the row windows of the two may not share memory
+    if (o && o_in->ptr == o->ptr) return LVX_ERR_SHAPE;
+    if (l_in == lse) return LVX_ERR_SHAPE;
+    if (o && o->ptr && s && row_count > 0 && s->B > 0 && s->Hq > 0) {
+        auto span = [&](const lvx_tensor* t, const char*& lo, const char*& hi) {
+            const int64_t last = (int64_t)(s->B - 1) * t->stride_b + (int64_t)(s->Hq - 1) * t->stride_h +
+                                 (int64_t)(row_begin + row_count - 1) * t->stride_s + s->D;
+            lo = static_cast<const char*>(t->ptr) + (int64_t)row_begin * t->stride_s * 2;
+            hi = static_cast<const char*>(t->ptr) + last * 2;
+        };
+        const char *alo, *ahi, *blo, *bhi;
+        span(o, alo, ahi);
+        span(o_in, blo, bhi);
+        if (alo < bhi && blo < ahi) return LVX_ERR_SHAPE;
+    }
+    if (lse && l_in && s && row_count > 0) {
+        const int64_t rows = (int64_t)s->B * s->Hq * s->Lq;
+        if (l_in < lse + rows && lse < l_in + rows) return LVX_ERR_SHAPE;
+    }
     return fwd_impl(s, q, k, v, o, lse, row_begin, row_count, kv_splits, workspace, workspace_bytes, stream,
                     o_in, l_in);
 }
@@ -378,7 +397,8 @@ static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_le
     const int wgs = s->B * s->Hq * tiles;
     const int blocks = (s->Lkv + 127) / 128;
     int ks = 1;
-    if (wgs <= 128) ks = std::min(std::min(8, 256 / wgs), blocks);
+    const int n_cu = cu_count();
+    if (wgs <= n_cu / 2) ks = std::min(std::min(8, n_cu / wgs), blocks);
     const int per = (blocks + ks - 1) / ks;
     *split_len = per * 128;
     return (blocks + per - 1) / per;

@@ -177,9 +177,11 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return r;
 }
 
-// Work-groups are dealt to the 8 XCDs round-robin by linear id.  Remap so that
+// Work-groups are dealt to the 8 XCDs of an MI355X round-robin by linear id.  Remap so that
 // each XCD receives one contiguous range of the work list: neighbours in the
-// list (which share K/V or Q tiles) then share that XCD's L2.
+// list (which share K/V or Q tiles) then share that XCD's L2.  A placement hint only: every id
+// below `total` is produced exactly once whatever the hardware does with it, so a device with
+// another XCD count computes the same results with less L2 sharing.
 __device__ __forceinline__ int xcd_remap(int bid, int total) {
     constexpr int NX = 8;
     int per = (total + NX - 1) / NX;

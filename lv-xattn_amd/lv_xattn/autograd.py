@@ -18,6 +18,7 @@ from typing import Callable, Optional
 import torch
 
 from . import ops
+from ._lib import LvxError
 from .attn import Mask, _attn_backward, _attn_forward, _reject_unsupported
 from .async_communication import reset_global_memory_buffer
 
@@ -141,9 +142,17 @@ def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = 
         # under autograd, on a detached x - and pushes dq, dk, dv back through it, so x gets its
         # gradient and so does whatever else run_function's graph reaches (projection weights,
         # norm weights, the visual states), where the reference returns none (:243).
+        # backward only runs when the output has a grad_fn, i.e. when x requires grad: with a frozen
+        # x (a frozen trunk under trainable projections) the parameters run_function reaches would
+        # silently get no gradient, so that case is refused while gradients are being recorded.
         @staticmethod
         def forward(ctx, x, run_function, is_causal):
             _reject_unsupported(is_causal)
+            if torch.is_grad_enabled() and not x.requires_grad:
+                raise LvxError("create_attention_class(...).apply(x, run_function, is_causal): x does not require "
+                               "grad, so backward would never run and run_function's parameters would get no "
+                               "gradient; pass x.requires_grad_() (its gradient can be discarded) or call under "
+                               "torch.no_grad()")
             q, k, v = run_function(x, get_global_cross_attention_states())
             sm_scale = q.size(-1) ** -0.5
             _, _, _, o, L = _attn_forward(q, k, v, is_causal, sm_scale, None, None, [], [], no_overlap,

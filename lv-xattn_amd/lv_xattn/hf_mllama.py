@@ -55,8 +55,11 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     Where a row does see a key, its masked positions become -inf: the result is the same
     (exp(-30000) is already 0 there) and the kernels can then skip whole tiles outside the span
     of the visible keys (ops.bias_hull), which is most of a Llama-3.2 mask."""
-    key = (mask.data_ptr(), mask._version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
-    if _bias_cache and _bias_cache[0] == key:
+    # an inference tensor (torch.inference_mode) has no version counter: its contents cannot be told
+    # apart from an edited copy at the same address, so it is converted every time and not kept
+    version = None if mask.is_inference() else mask._version
+    key = (mask.data_ptr(), version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
+    if version is not None and _bias_cache and _bias_cache[0] == key:
         return _bias_cache[1]
     m = mask.float()
     masked = m <= -30000.0
@@ -64,7 +67,8 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     bias = torch.where(masked & sees_a_key, float("-inf"), m.clamp_min(-30000.0))
     # every cross-attention layer of a model gets the same mask, in forward and again in backward:
     # the last conversion is kept (with the mask itself, so that its address cannot be reused)
-    _bias_cache[:] = [key, bias, mask]
+    if version is not None:
+        _bias_cache[:] = [key, bias, mask]
     return bias
 
 

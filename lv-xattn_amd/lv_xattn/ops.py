@@ -65,14 +65,17 @@ def _shape(q: torch.Tensor, k: torch.Tensor, scale: float, mask: Optional[Mask],
         if (bias.dtype != torch.float32 or bias.dim() != 4 or bias.device != q.device or bias.stride(3) != 1
                 or bias.shape[0] not in (1, B) or bias.shape[1] not in (1, Hq) or tuple(bias.shape[2:]) != (Lq, Lkv)):
             raise LvxError(f"bias must be an fp32 [B|1, Hq|1, {Lq}, {Lkv}] tensor with unit last stride on {q.device}")
-        if bias.stride(2) < (Lkv + 3) // 4 * 4:
+        # a dimension of extent 1 is never stepped over: whatever stride torch reports for it, the
+        # library is told the value its own checks accept (0 to broadcast, the padded row length)
+        row_stride = bias.stride(2) if Lq > 1 else (Lkv + 3) // 4 * 4
+        if row_stride < (Lkv + 3) // 4 * 4:
             raise LvxError("bias rows must be padded to a multiple of 4 floats (row stride >= Lkv rounded up to 4)")
-        if bias.data_ptr() % 16 or any(bias.stride(i) % 4 and bias.shape[i] > 1 for i in range(3)):
+        if bias.data_ptr() % 16 or row_stride % 4 or any(bias.stride(i) % 4 and bias.shape[i] > 1 for i in range(2)):
             raise LvxError("bias must be 16-byte aligned with batch, head and row strides that are multiples of 4 floats")
         s.bias = bias.data_ptr()
         s.bias_stride_b = bias.stride(0) if bias.shape[0] > 1 else 0
         s.bias_stride_h = bias.stride(1) if bias.shape[1] > 1 else 0
-        s.bias_stride_r = bias.stride(2)
+        s.bias_stride_r = row_stride
     return s
 
 

@@ -39,7 +39,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_version_and_error_strings(lib):
-    assert lib.lvx_version() == 100
+    assert lib.lvx_version() == 101
     assert lib.lvx_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert lib.lvx_strerror(code) not in (b"", b"unknown lvx error")
@@ -113,7 +113,14 @@ def test_other_entry_points_reject_bad_arguments(lib):
                            0x2000, 0, 64, 1, None, 0, None) == -2
     assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, C.byref(t), 0x2000,
                            0, 64, 1, None, 0, None) == -3
+    # ... nor may the accumulator's LSE be the output's, or the two O windows overlap at another base
     assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(o_in), 0x2000, C.byref(t), 0x2000,
+                           0, 64, 1, None, 0, None) == -3
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(o_in), 0x2100, C.byref(t), 0x2000,
+                           0, 64, 1, None, 0, None) == -3
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(_t(ptr=0x1100)), 0x800000,
+                           C.byref(t), 0x2000, 0, 64, 1, None, 0, None) == -3
+    assert lib.lvx_fwd_acc(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(o_in), 0x800000, C.byref(t), 0x2000,
                            0, 0, 1, None, 0, None) == 0          # no rows: accepted, nothing launched
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, None, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, 1 << 30, None) == -1
@@ -216,5 +223,5 @@ def test_plain_c_caller_compiles_against_the_header_and_calls_the_library(lib, t
     r = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     version, rc, msg, ws = r.stdout.strip().split("|")
-    assert int(version) == 100 and int(rc) == -4 and msg == "head_dim must be 128"
+    assert int(version) == 101 and int(rc) == -4 and msg == "head_dim must be 128"
     assert int(ws) == 4 * 8 * 64 * (128 * 2 + 4)

@@ -148,3 +148,26 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "single-GPU" in (r.stderr + r.stdout)
+
+
+def test_mask_conversion_of_the_hf_hook_under_inference_mode():
+    """An inference tensor has no version counter: the converted mask is then rebuilt on every call
+    instead of being kept, and no error is raised."""
+    from lv_xattn import hf_mllama
+    hf_mllama.clear_mask_cache()
+    neg = torch.finfo(torch.bfloat16).min
+    with torch.inference_mode():
+        mask = torch.zeros(1, 1, 3, 8, dtype=torch.bfloat16)
+        mask[0, 0, 1, 4:] = neg
+        b1 = hf_mllama._mask_bias(mask)
+        assert b1.dtype == torch.float32 and b1[0, 0, 1, 4:].eq(float("-inf")).all() and b1[0, 0, 1, :4].eq(0).all()
+        mask[0, 0, 2, :2] = neg                   # edited in place: no version tells, so nothing may be reused
+        b2 = hf_mllama._mask_bias(mask)
+        assert b2[0, 0, 2, :2].eq(float("-inf")).all()
+    assert not hf_mllama._bias_cache
+    # an ordinary tensor is kept until it changes
+    mask = torch.zeros(1, 1, 3, 8, dtype=torch.bfloat16)
+    assert hf_mllama._mask_bias(mask) is hf_mllama._mask_bias(mask)
+    mask[0, 0, 0, 0] = neg
+    assert hf_mllama._mask_bias(mask)[0, 0, 0, 0] == float("-inf")
+    hf_mllama.clear_mask_cache()

@@ -1,11 +1,14 @@
 """lvx_fwd_noalloc - the forward entry point whose key-split partials live in an array inside
 the library instead of a caller's workspace - against lvx_fwd on the same inputs, through the
 C ABI: two calls in a row, the second on a smaller input (the array keeps the first call's
-contents), bit for bit; then the size limit."""
+contents), bit for bit, and against the CPU oracle; then the size limit."""
 import ctypes as C
 
 import pytest
 import torch
+
+from oracle import lvx_oracle as orc
+from parity import check_lse, check_o
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -50,6 +53,10 @@ def test_noalloc_forward_matches_forward_twice_then_rejects_what_does_not_fit():
     o, l, o_ref, l_ref = _both(ops, q2, k2, v2, 2, 0, 96)
     assert torch.equal(o, o_ref) and torch.equal(l, l_ref)
     assert o.abs().max() > 0
+    # and on its own feet: the second call against the CPU oracle (full softmax in fp32)
+    o_orc, l_orc = orc.attention_dense(q2.float().cpu(), k2.float().cpu(), v2.float().cpu(), 128 ** -0.5)
+    check_o(o, o_orc, "O of lvx_fwd_noalloc")
+    check_lse(l, l_orc, "LSE of lvx_fwd_noalloc")
 
     # one split needs no array at all
     o, l, o_ref, l_ref = _both(ops, q, k, v, 1, 0, 256)
