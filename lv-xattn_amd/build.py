@@ -56,7 +56,9 @@ def _run(cmd, verbose):
 # hand-scheduled inner loops: (generator, arguments, include file it writes)
 GENERATED = [("gen_fwd_loop.py", ["bf16"], "lvx_fwd_loop_bf16.inc"),
              ("gen_bwd_loop.py", ["p"], "lvx_bwd_loop_p.inc"),
-             ("gen_bwd_loop.py", ["d"], "lvx_bwd_loop_d.inc")]
+             ("gen_bwd_loop.py", ["d"], "lvx_bwd_loop_d.inc"),
+             ("gen_gemm_loop.py", ["bp"], "lvx_gemm_loop_bp.inc"),
+             ("gen_gemm_loop.py", ["bt"], "lvx_gemm_loop_bt.inc")]
 
 
 def generate() -> None:

@@ -31,6 +31,9 @@ namespace lvx {
 
 namespace {
 
+// registers the hand-scheduled loop uses besides its operands (see gen_gemm_loop.py)
+#define LVX_GEMM_LOOP_CLOBBERS "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223"
+
 constexpr int BK = 32;                 // contraction depth of one stage
 __device__ uint32_t zero_chunk[4];     // source of the chunks past the end of a contraction
 
@@ -110,8 +113,6 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     constexpr int LPG_A = RA::CHUNKS / 8;
     static_assert(RA::CHUNKS % 8 == 0 && RB::CHUNKS % 8 == 0, "chunks split evenly over 8 waves");
     constexpr int NRA = RA::NRD(WM), NRB = RB::NRD(WN);
-    // LDS read instructions per MFMA of a stage (a transposing operand read is two)
-    constexpr int LDS_PER_MFMA = (2 * (WM * (A_MCONTIG ? 2 : 1) + WN * (B_NCONTIG ? 2 : 1)) + 2 * WM * WN - 1) / (2 * WM * WN);
     __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
     const int wid0 = xcd_remap(blockIdx.x, p.total_wg);
@@ -214,56 +215,53 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-#ifdef LVX_GEMM_PIPE
-    // Every wave software-pipelines by itself: the operands of stage s+1 are read from LDS into a second
-    // register set while the 16 MFMAs of stage s issue, one barrier per stage.
-    bf16x8 am[2][2][WM], bn[2][2][WN];      // [register set][k-step][tile]
-#pragma unroll
-    for (int s = 0; s < NS - 1; ++s)
-        if (s < steps) issue(s);
-    if (steps > NS - 2) wait_vmcnt<(NS - 2) * LPG>();
-    else wait_vmcnt<0>();
-    phase_barrier();
-    auto fetch = [&](auto set_c, int s) __attribute__((always_inline)) {
-        constexpr int RS = decltype(set_c)::value;
-        const uint32_t base = (uint32_t)(s % NS) * STAGE;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-            for (int t = 0; t < WM; ++t) am[RS][kk][t] = RA::operand(lds, base, rda, t, kk);
-#pragma unroll
-            for (int t = 0; t < WN; ++t) bn[RS][kk][t] = RB::operand(lds, base + RA::BYTES, rdb, t, kk);
+    // The 256 x 256 bf16 tile with A stored [m][k] and whole stages only (the K/V projection and
+    // dX_vis) takes the hand-scheduled loop of gen_gemm_loop.py, one run per contraction segment; every
+    // other case takes the ping-pong loop below.
+    constexpr bool FAST = !F16 && !A_MCONTIG && GM == 2 && GN == 4 && WM == 4 && WN == 2 && NS == 4;
+    if constexpr (FAST) {
+        const int st0 = klen0 / BK, st1 = klen1 / BK;
+        const bool whole = klen0 % BK == 0 && klen1 % BK == 0 && st0 % 4 == 0 && st1 % 4 == 0 && st0 >= 8 &&
+                           (st1 == 0 || st1 >= 8);
+        if (whole) {
+            uint32_t ra[4], rb[4];
+            ra[0] = lds0 + rda[0]; ra[1] = lds0 + rda[1]; ra[2] = ra[0] + 65536u; ra[3] = ra[1] + 65536u;
+            rb[0] = lds0 + rdb[0]; rb[1] = lds0 + rdb[1]; rb[2] = rb[0] + 65536u; rb[3] = rb[1] + 65536u;
+            const uint32_t lds_w = uniform32(lds0 + (uint32_t)wave * 1024u);
+            for (int sg = 0; sg < (st1 ? 2 : 1); ++sg) {
+                const int nst = sg ? st1 : st0;
+                const char* ap = uniform_ptr(abase[sg] + (int64_t)(sg ? 0 : s_lo) * a_kstride);
+                const char* bp = uniform_ptr(bbase[sg] + (int64_t)(sg ? 0 : s_lo) * b_kstride);
+                int trips = uniform32(nst / 4), todo = uniform32(nst);
+                __syncthreads();     // the stage buffers are free
+                if (B_NCONTIG) {
+                    asm volatile(
+#include "lvx_gemm_loop_bt.inc"
+                        : "+{v[0:15]}"(acc[0][0]), "+{v[16:31]}"(acc[0][1]), "+{v[32:47]}"(acc[0][2]), "+{v[48:63]}"(acc[0][3]),
+                          "+{v[64:79]}"(acc[1][0]), "+{v[80:95]}"(acc[1][1]), "+{v[96:111]}"(acc[1][2]), "+{v[112:127]}"(acc[1][3]),
+                          "+{s[44:45]}"(ap), "+{s[46:47]}"(bp), "+{s51}"(trips), "+{s52}"(todo)
+                        : "{v224}"(ra[0]), "{v225}"(ra[1]), "{v226}"(ra[2]), "{v227}"(ra[3]),
+                          "{v228}"(rb[0]), "{v229}"(rb[1]), "{v230}"(rb[2]), "{v231}"(rb[3]),
+                          "{v232}"(voff[0]), "{v233}"(voff[1]), "{v234}"(voff[2]), "{v235}"(voff[3]),
+                          "{s48}"(uniform32((uint32_t)a_kstride)), "{s49}"(uniform32((uint32_t)b_kstride)), "{s50}"(lds_w)
+                        : "memory", "vcc", "scc", "m0", "s53", "s54", "s55", LVX_GEMM_LOOP_CLOBBERS);
+                } else {
+                    asm volatile(
+#include "lvx_gemm_loop_bp.inc"
+                        : "+{v[0:15]}"(acc[0][0]), "+{v[16:31]}"(acc[0][1]), "+{v[32:47]}"(acc[0][2]), "+{v[48:63]}"(acc[0][3]),
+                          "+{v[64:79]}"(acc[1][0]), "+{v[80:95]}"(acc[1][1]), "+{v[96:111]}"(acc[1][2]), "+{v[112:127]}"(acc[1][3]),
+                          "+{s[44:45]}"(ap), "+{s[46:47]}"(bp), "+{s51}"(trips), "+{s52}"(todo)
+                        : "{v224}"(ra[0]), "{v225}"(ra[1]), "{v226}"(ra[2]), "{v227}"(ra[3]),
+                          "{v228}"(rb[0]), "{v229}"(rb[1]), "{v230}"(rb[2]), "{v231}"(rb[3]),
+                          "{v232}"(voff[0]), "{v233}"(voff[1]), "{v234}"(voff[2]), "{v235}"(voff[3]),
+                          "{s48}"(uniform32((uint32_t)a_kstride)), "{s49}"(uniform32((uint32_t)b_kstride)), "{s50}"(lds_w)
+                        : "memory", "vcc", "scc", "m0", "s53", "s54", "s55", LVX_GEMM_LOOP_CLOBBERS);
+                }
+            }
+            goto epilogue;
         }
-    };
-    auto stage = [&](auto set_c, int s) __attribute__((always_inline)) {
-        constexpr int RS = decltype(set_c)::value;
-        // stage s+1 has landed (this wave's chunks: vmcnt; everyone's: barrier); every wave has read stage s-1
-        if (s + NS - 2 < steps) wait_vmcnt<(NS - 3) * LPG>();
-        else wait_vmcnt<0>();
-        wait_lds();
-        __builtin_amdgcn_s_barrier();
-        if (s + NS - 1 < steps) issue(s + NS - 1);
-        if (s + 1 < steps) fetch(std::integral_constant<int, RS ^ 1>{}, s + 1);
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-            for (int nt = 0; nt < WN; ++nt)
-#pragma unroll
-                for (int mt = 0; mt < WM; ++mt) acc[nt][mt] = E::mfma(bn[RS][kk][nt], am[RS][kk][mt], acc[nt][mt]);
-        // spread the MFMAs over the LDS reads and the global loads
-#pragma unroll
-        for (int i = 0; i < 2 * WM * WN; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, LDS_PER_MFMA, 0);   // LDS reads
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a vector-memory read, while there are any
-        }
-    };
-    fetch(std::integral_constant<int, 0>{}, 0);
-    for (int s = 0; s < steps; s += 2) {
-        stage(std::integral_constant<int, 0>{}, s);
-        if (s + 1 < steps) stage(std::integral_constant<int, 1>{}, s + 1);
     }
-#else
+
     // prologue: stages 0 .. NS-2 in flight, stage 0 landed
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s)
@@ -308,8 +306,7 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     }
     if (set == 0) phase_barrier();
 
-#endif
-
+epilogue:
     // C^T tile: accumulator rows = n, cols = m
     if (nks > 1) {   // partial tile of a split contraction: fp32, into this split's slice
         float* const C32 = p.c32 + ksp * p.c32_split + (int64_t)z * p.c32_batch;
