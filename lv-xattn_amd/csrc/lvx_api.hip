@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 using namespace lvx;
@@ -120,6 +121,19 @@ size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count, int32
     return (size_t)kv_splits * rows * (s->D * sizeof(uint16_t) + sizeof(float));
 }
 
+static int cu_count();
+
+// Whether the forward runs in its wide form (a wave owns 64 rows and its SIMD; one work-group per
+// CU): bf16 without a dense bias or an interval mask, whole 64-row blocks, and enough work-groups
+// that every CU has one.
+static bool fwd_wide(const lvx_attn_shape* s, int32_t row_count, int rs, int kv_splits) {
+    if (const char* e = getenv("LVX_FWD_WIDE")) return atoi(e) != 0 && s->dtype == LVX_BF16 && !s->bias;
+    if (s->dtype != LVX_BF16 || s->bias || s->kv_start) return false;
+    if (row_count % (64 * rs) != 0) return false;
+    const int64_t wgs = (int64_t)s->B * (s->Hq / (4 / rs)) * (row_count / (64 * rs)) * kv_splits;
+    return wgs >= cu_count();
+}
+
 // lvx_fwd, and lvx_fwd_acc when (o_in, l_in) is given: the result is then merged with that
 // incoming accumulator before it is written to (o, lse).
 static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, const lvx_tensor* v,
@@ -149,7 +163,9 @@ static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tens
     p.HG = gcd(p.G, 4);
     p.RS = 4 / p.HG;
     p.row_begin = row_begin; p.row_end = row_begin + row_count;
-    p.n_row_tiles = (row_count + 32 * p.RS - 1) / (32 * p.RS);
+    p.wide = fwd_wide(s, row_count, p.RS, kv_splits) ? 1 : 0;
+    const int wg_rows = (p.wide ? 64 : 32) * p.RS;
+    p.n_row_tiles = (row_count + wg_rows - 1) / wg_rows;
     p.n_head_groups = s->Hq / p.HG;
     p.scale = s->scale; p.scale_log2e = s->scale * LOG2E;
 

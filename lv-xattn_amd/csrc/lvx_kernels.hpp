@@ -37,7 +37,8 @@ struct FwdParams {
     int B, Hq, Hkv, Lq, Lkv;
     int G;                     // q heads per kv head
     int HG;                    // q heads a work-group covers (one per wave)
-    int RS;                    // 32-row sub-tiles a work-group covers per head
+    int RS;                    // row sub-tiles a work-group covers per head
+    int wide;                  // 1: a wave owns 64 rows (two blocks of 32) instead of 32; bf16 without bias only
     int row_begin, row_end;
     int n_row_tiles, n_head_groups, nsplit, split_len, total_wg;
     float scale, scale_log2e;

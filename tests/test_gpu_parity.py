@@ -265,8 +265,19 @@ def test_preprocess_delta(lvx):
 
 
 # ------------------------------------------------------------------ forward
+@pytest.fixture(params=["auto", "wide"])
+def form(request, monkeypatch):
+    """The forward kernel has two forms: a wave owns 32 rows, or 64 rows and its SIMD (picked for bf16
+    launches without mask or bias that give every CU a work-group).  'wide' forces the second on
+    these small shapes - also with masks, ragged row counts and key splits - through the
+    environment variable the library reads at every call."""
+    if request.param == "wide":
+        monkeypatch.setenv("LVX_FWD_WIDE", "1")
+    return request.param
+
+
 @pytest.mark.parametrize("mode", ["rounds", "batched", "splits"])
-def test_forward_cfg1s(lvx, mode):
+def test_forward_cfg1s(lvx, mode, form):
     w = orc.make_inputs(orc.workload("cfg1s"))
     t = w.tensors
     o_ref, l_ref = orc.round_loop_forward(t["q"], t["k"], t["v"], w.scale, w.rounds)
@@ -285,7 +296,7 @@ def test_forward_cfg1s(lvx, mode):
 @pytest.mark.parametrize("kw", [dict(), dict(kv_splits=1), dict(kv_splits=4), dict(batched=True),
                                 dict(batched=True, kv_splits=3)],
                          ids=["auto", "nosplit", "split4", "batched", "batched_split3"])
-def test_forward_with_incoming_accumulator(lvx, kw):
+def test_forward_with_incoming_accumulator(lvx, kw, form):
     # lvx_fwd_acc: the round's partial and the travelling accumulator leave as one result; with
     # key splits one merge launch folds the splits and the accumulator, which may hold NaN
     # where its LSE is -inf (nothing folded in yet)
@@ -329,7 +340,7 @@ def test_forward_kv_chunks_then_merge_equals_full_softmax(lvx):
     check_lse(l_acc, l_ref)
 
 
-def test_forward_masked_ragged_cfg4s(lvx):
+def test_forward_masked_ragged_cfg4s(lvx, form):
     w = orc.make_inputs(orc.workload("cfg4s"))
     t = w.tensors
     allowed = orc.workload_allowed(w)
@@ -344,7 +355,7 @@ def test_forward_masked_ragged_cfg4s(lvx):
         assert (o.float().cpu()[dead] == 0).all()
 
 
-def test_forward_kv_len_only(lvx):
+def test_forward_kv_len_only(lvx, form):
     w = orc.make_inputs(orc.workload("cfg4s"))
     t = w.tensors
     w.tensors = {k_: v_ for k_, v_ in t.items() if not k_.startswith("kv_")}
@@ -358,7 +369,7 @@ def test_forward_kv_len_only(lvx):
     check_lse(L, l_ref)
 
 
-def test_forward_mha_and_gqa8_strided_inputs(lvx):
+def test_forward_mha_and_gqa8_strided_inputs(lvx, form):
     # G = 1 (one head x 128 rows per work-group) and G = 8 (two groups per kv head);
     # q/k/v given as [B,S,H,D]-memory views, as a fused projection would produce them
     g = torch.Generator().manual_seed(21)
