@@ -26,6 +26,7 @@ P-waves: v[168:175] P packed   v[176:191] LSE*log2(e) of 16 rows   v[192:199] dS
   s[54:55] / s[56:57] / s[60:61] what a head change adds to the Q / dO / workspace address
   s62 LDS address of this wave's part of Q buffer 0   s63 of the metadata records   s64 trips
   s65 1 in wave 0 (it requests the metadata)   s[66:77] workspace addresses of the tiles in flight
+  s[78:79] scratch
 D-waves: v[168:175] P handed over   v[176:183] dS packed   v[184:199] delta*scale of 16 rows
   v216 P hand-over read address   v217 metadata read address   v218 dS^T staging write address
 """
@@ -63,10 +64,15 @@ def sr(base, n=1):
 class Stream:
     """Instruction list with a model of the in-order LDS queue for s_waitcnt lgkmcnt."""
 
-    def __init__(self):
+    def __init__(self, seed=None):
         self.out = []
         self.n_lds = 0
         self.tag = {}
+        self.done = 0           # LDS operations 1 .. done are known to have completed
+        self.last_write = 0     # position of the last ds_write
+        if seed is not None:    # what the step before left in flight: see carry_over()
+            self.n_lds = seed["n"]
+            self.tag = dict(seed["tag"])
 
     def emit(self, s):
         if "nodma" in OPTS and (s.startswith("global_load_lds") or s.startswith("s_add_i32 m0")):
@@ -89,10 +95,26 @@ class Stream:
         self.n_lds += 1
         if tag is not None:
             self.tag[tag] = self.n_lds
+        if text is not None and text.startswith("ds_write"):
+            self.last_write = self.n_lds
 
     def wait(self, tag):
-        n = self.n_lds - self.tag[tag]
-        self.out.append(f"s_waitcnt lgkmcnt({min(n, 15)})")
+        if self.tag[tag] <= self.done:      # an earlier wait of this step covers it
+            return
+        n = min(self.n_lds - self.tag[tag], 15)
+        self.out.append(f"s_waitcnt lgkmcnt({n})")
+        self.done = self.n_lds - n
+
+    def carry_over(self, u_next):
+        """What a step leaves to the next one: the LDS operations it issued after its last write (the
+        next step waits at its top until only these are in flight: LDS operations complete in order, so
+        the writes other waves are about to read have then landed) and, among them, the reads of the
+        first operands of the next step."""
+        n = self.n_lds - self.last_write
+        tag = {t: pos - self.last_write for t, pos in self.tag.items()     # <= 0: read before the write
+               if isinstance(t, tuple) and t[0] == "op" and t[1] == u_next}
+        assert len(tag) == AHEAD and n <= 15, (n, tag)
+        return {"n": n, "tag": tag}
 
     def wait_needed(self, tag):
         return self.n_lds - self.tag[tag]
@@ -155,16 +177,16 @@ def flat(items):
     return out
 
 
-def p_step(u):
+def p_step(u, seed):
     """P-wave step i, i % 6 == (u + 3) % 6.  Operands 0..6 were read in the step before."""
-    st = Stream()
+    st = Stream(seed)
     e = st.emit
     sl_p = (u + 2) % 6
     par = u & 1                                                  # (i + 1) & 1: P(i-1) hand-over, dS^T(i-3)
     carry, new = SET[u & 1], SET[(u + 1) & 1]
-    # tile i+1 has landed: after its loads this wave issued 2 stores and 4 (wave 0: 5) loads
-    e("s_waitcnt vmcnt(6)")
-    e("s_waitcnt lgkmcnt(0)")
+    # tile i+1 has landed: after its loads this wave issued 2 stores, 4 (wave 0: 5) loads and 2 stores
+    e("s_waitcnt vmcnt(6)" if "storefirst" in OPTS else "s_waitcnt vmcnt(8)")
+    e(f"s_waitcnt lgkmcnt({st.n_lds})")
     e("s_barrier")
     for vg in range(4):
         st.lds(f"ds_read_b128 {vr(LSE + 4 * vg, 4)}, v{A_META} offset:{sl_p * META_SZ + vg * 32}", ("lse", vg))
@@ -190,25 +212,30 @@ def p_step(u):
     valu.append(lambda: st.lds(f"ds_write_b128 v{A_PB}, {vr(PU, 4)} offset:{par * PB_SZ}"))
     valu.append(lambda: st.lds(f"ds_write_b128 v{A_PB}, {vr(PU + 4, 4)} offset:{par * PB_SZ + 1024}"))
 
-    # second half: dS^T(i-3) copy-out, request of tile i+3, the walk
+    # second half: request of tile i+3 and the walk, dS^T(i-3) copy-out.  The loads go first: the wait
+    # at the top of a step then leaves the two stores of the step before last in flight as well
     tail = []
     tail.append(lambda: st.lds(f"ds_read_b128 {vr(CPD, 4)}, v{A_CP} offset:{par * DST_SZ}", "cp0"))
     tail.append(lambda: st.lds(f"ds_read_b128 {vr(CPD + 4, 4)}, v{A_CP} offset:{par * DST_SZ + 5120}", "cp1"))
     ws_old = 66 + 2 * (u % 6)          # workspace address of tile i-3 (tile i+3 takes its place below)
-    tail.append(lambda: st.wait("cp0"))
-    tail.append(f"global_store_dwordx4 v{G_CP0}, {vr(CPD, 4)}, {sr(ws_old, 2)}")
-    tail.append(lambda: st.wait("cp1"))
-    tail.append(f"global_store_dwordx4 v{G_CP1}, {vr(CPD + 4, 4)}, {sr(ws_old, 2)}")
     fetch = p_fetch(u, 3)
     if u == 5:      # the last step of the last trip requests nothing: the steps after the loop do
         fetch = [["s_cmp_eq_u32 s64, 1", "s_cbranch_scc1 LVX_BWD_NOFETCH_%="] + flat(fetch) + ["LVX_BWD_NOFETCH_%=:"]]
-    tail += fetch
+    store = [lambda: st.wait("cp0"), f"global_store_dwordx4 v{G_CP0}, {vr(CPD, 4)}, {sr(ws_old, 2)}",
+             lambda: st.wait("cp1"), f"global_store_dwordx4 v{G_CP1}, {vr(CPD + 4, 4)}, {sr(ws_old, 2)}"]
+    if "storefirst" in OPTS:
+        tail += store + fetch
+    else:
+        # the stores read the workspace address of tile i-3 before the walk overwrites it: keep a copy
+        tail += [f"s_mov_b64 s[78:79], {sr(ws_old, 2)}"] + fetch
+        store[1] = f"global_store_dwordx4 v{G_CP0}, {vr(CPD, 4)}, s[78:79]"
+        store[3] = f"global_store_dwordx4 v{G_CP1}, {vr(CPD + 4, 4)}, s[78:79]"
+        tail += store
 
     mf = []
     for k in range(16):
         def m(k=k):
-            if k >= AHEAD:
-                st.wait(("op", u, k))
+            st.wait(("op", u, k))
             slot = STG + 4 * (k % NSLOT)
             if k < 8:
                 c = "0" if k == 0 else vr(new, 16)
@@ -226,7 +253,7 @@ def p_step(u):
     nt = sum(len(x) if isinstance(x, list) else 1 for x in tail)
     shares = [(nv + 7) // 8] * 8 + [(nt + 6) // 7] * 8
     spread(st, mf, side, shares)
-    return st.out
+    return st.out, st.carry_over((u + 1) % 6)
 
 
 def p_prologue():
@@ -239,6 +266,7 @@ def p_prologue():
         p_read_op(st, 0, n)
     for y in flat(p_fetch(0, 2)):
         st.emit(y)
+    st.emit("s_waitcnt lgkmcnt(0)")     # the first step counts on no more in flight than a step leaves
     return st.out
 
 
@@ -255,14 +283,14 @@ def d_read_op(st, u, n):
         st.lds(f"ds_read_b64_tr_b16 {vr(slot + 2, 2)}, v{TA + 2 * dt + 1} offset:{off}", ("op", u, n))
 
 
-def d_step(u):
+def d_step(u, seed):
     """D-wave step i, i % 6 == (u + 3) % 6.  Operands 0..6 were read in the step before."""
-    st = Stream()
+    st = Stream(seed)
     e = st.emit
     sl_pp = (u + 1) % 6                        # buffer of tile i-2 (Q^T, metadata)
     par = (u + 1) & 1                          # i & 1: P(i-2) hand-over, dS^T(i-2) staging
     carry, new = SET[u & 1], SET[(u + 1) & 1]
-    e("s_waitcnt lgkmcnt(0)")
+    e(f"s_waitcnt lgkmcnt({st.n_lds})")
     e("s_barrier")
     st.lds(f"ds_read_b128 {vr(PU, 4)}, v{A_PB} offset:{par * PB_SZ}", ("pu", 0))
     st.lds(f"ds_read_b128 {vr(PU + 4, 4)}, v{A_PB} offset:{par * PB_SZ + 1024}", ("pu", 1))
@@ -292,8 +320,7 @@ def d_step(u):
     mf = []
     for k in range(16):
         def m(k=k):
-            if k >= AHEAD:
-                st.wait(("op", u, k))
+            st.wait(("op", u, k))
             slot = STG + 4 * (k % NSLOT)
             if k < 8:
                 c = "0" if k == 0 else vr(new, 16)
@@ -308,7 +335,7 @@ def d_step(u):
         mf.append(m)
     shares = [6] * 8 + [4, 4, 4, 2, 2, 2, 0, 0]
     spread(st, mf, valu, shares)
-    return st.out
+    return st.out, st.carry_over((u + 1) % 6)
 
 
 def d_prologue():
@@ -317,6 +344,7 @@ def d_prologue():
     st.emit("s_barrier")
     for n in range(AHEAD):
         d_read_op(st, 0, n)
+    st.emit("s_waitcnt lgkmcnt(0)")     # the first step counts on no more in flight than a step leaves
     return st.out
 
 
@@ -368,9 +396,15 @@ def check(ins):
 
 def main():
     step = p_step if ROLE == "p" else d_step
+    # what step 5 leaves to step 0 of the next trip: every step issues the same LDS operations in the
+    # same order, so a dry run of one step tells
+    _, seed = step(5, {"n": AHEAD, "tag": {("op", 5, k): k + 1 for k in range(AHEAD)}})
     body = []
     for u in range(6):
-        body += [x for x in step(u) if x is not None]
+        ins, left = step(u, seed)
+        assert u == 5 or left == {"n": seed["n"], "tag": {("op", u + 1, t[2]): p for t, p in seed["tag"].items()}}, (left, seed)
+        seed = left
+        body += [x for x in ins if x is not None]
     check(body + body)
     cnt = "s64"
     lines = (p_prologue() if ROLE == "p" else d_prologue()) + ["LVX_BWD_LOOP_%=:"] + body + [f"s_sub_i32 {cnt}, {cnt}, 1", f"s_cmp_lg_u32 {cnt}, 0", "s_cbranch_scc1 LVX_BWD_LOOP_%=",

@@ -537,7 +537,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                           "{s40}"(uniform32(c)), "{s41}"(uniform32((uint32_t)BM * qrow_b)), "{s42}"(uniform32((uint32_t)BM * dorow_b)), "{s53}"(uniform32(n_qtiles)),
                           "{s[54:55]}"(hdq), "{s[56:57]}"(hddo), "{s[60:61]}"(hdws),
                           "{s62}"(uniform32(lds0 + (uint32_t)slice * 2048u)), "{s63}"(uniform32(meta0)), "{s65}"(uniform32(wave == 0 ? 1 : 0))
-                        : "memory", "vcc", "scc", "m0", LVX_BWD_LOOP_CLOBBERS);
+                        : "memory", "vcc", "scc", "m0", "s78", "s79", LVX_BWD_LOOP_CLOBBERS);
                     wait_vmcnt<0>();    // the steps below count the operations in flight from scratch
                     w_q[0] = reinterpret_cast<const uint16_t*>(w0) - ws_k;
                     w_q[1] = reinterpret_cast<const uint16_t*>(w1) - ws_k;
