@@ -284,6 +284,10 @@ def other_workload(name, torch, dev, steps=10, warmup=5):
         other = Layer(w, "rounds", dev)
         fns = {"batched": layer.step, "rounds": other.step}
     rec["flops_per_step"] = step_flops
+    if fwd_only:
+        # a step here is a few hundred microseconds: time enough of them to get past the clock
+        # management's first milliseconds under load, as the longer workloads do by themselves
+        steps, warmup = 5 * steps, 8 * warmup
     for mode, fn in fns.items():
         ms = time_gpu(fn, steps, warmup, torch)
         rec[mode] = {"ms_per_step": round(ms, 4), "tflops": round(step_flops / ms / 1e9, 2),
