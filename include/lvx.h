@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define LVX_VERSION 101
+#define LVX_VERSION 102
 
 #define LVX_OK 0
 #define LVX_ERR_NULL (-1)        /* a required pointer is NULL */
@@ -158,6 +158,19 @@ int lvx_merge(const lvx_attn_shape* shape, const lvx_tensor* o_acc, float* l_acc
  * a mask handed over as a bias cost what it leaves visible.
  */
 int lvx_bias_hull(const lvx_attn_shape* shape, int32_t* kv_start, int32_t* kv_end, void* stream);
+
+/*
+ * Tests whether shape->bias is nothing but the interval mask lvx_bias_hull found for it:
+ * *not_interval (device memory, zero on entry) is set to 1 when some entry inside a row's
+ * [kv_start, kv_end) is not exactly 0 (outside the hull every entry is -inf by construction).
+ * When it stays 0 the caller may drop the bias and run lvx_fwd / lvx_bwd with the intervals
+ * alone - the interval-mask kernels, which read no bias at all - and get the same result.
+ * No counterpart in the reference (lv_xattn/attn.py:238-241 adds whatever bias it is handed);
+ * this is what lets a Llama-3.2 cross-attention mask that arrives dense, as transformers
+ * builds it, run at the cost of the compact mask.
+ */
+int lvx_bias_is_interval(const lvx_attn_shape* shape, const int32_t* kv_start, const int32_t* kv_end,
+                         int32_t* not_interval, void* stream);
 
 /*
  * delta[b*Hq+h, row] = sum_d O * dO.  Replaces `_bwd_preprocess_do_o_dot`

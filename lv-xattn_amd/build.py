@@ -55,7 +55,7 @@ def _run(cmd, verbose):
 
 # hand-scheduled inner loops: (generator, arguments, include file it writes)
 GENERATED = [("gen_fwd_loop.py", ["bf16"], "lvx_fwd_loop_bf16.inc"),
-    ("gen_fwd_loop_wide.py", [], "lvx_fwd_loop_wide.inc"),
+             ("gen_fwd_loop_wide.py", [], "lvx_fwd_loop_wide.inc"),
              ("gen_bwd_loop.py", ["p"], "lvx_bwd_loop_p.inc"),
              ("gen_bwd_loop.py", ["d"], "lvx_bwd_loop_d.inc"),
              ("gen_gemm_loop.py", ["bp"], "lvx_gemm_loop_bp.inc"),

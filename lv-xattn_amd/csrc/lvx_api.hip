@@ -331,6 +331,18 @@ int lvx_bias_hull(const lvx_attn_shape* s, int32_t* kv_start, int32_t* kv_end, v
     return static_cast<int>(launch_bias_hull(p, static_cast<hipStream_t>(stream)));
 }
 
+int lvx_bias_is_interval(const lvx_attn_shape* s, const int32_t* kv_start, const int32_t* kv_end, int32_t* not_interval,
+                         void* stream) {
+    LVX_TRY(check_shape(s));
+    if (!s->bias || !kv_start || !kv_end || !not_interval) return LVX_ERR_NULL;
+    BiasHullParams p{};
+    p.bias = s->bias; p.bias_b = s->bias_stride_b; p.bias_h = s->bias_stride_h; p.bias_r = s->bias_stride_r;
+    p.kv_start = const_cast<int32_t*>(kv_start); p.kv_end = const_cast<int32_t*>(kv_end);
+    p.B = s->B; p.heads = s->bias_stride_h ? s->Hq : 1; p.Lq = s->Lq; p.Lkv = s->Lkv;
+    p.flag = not_interval;
+    return static_cast<int>(launch_bias_interval(p, static_cast<hipStream_t>(stream)));
+}
+
 int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_tensor* dout, float* delta,
                        int32_t row_begin, int32_t row_count, void* stream) {
     LVX_TRY(check_shape(s));

@@ -70,11 +70,13 @@ struct MergeParams {
 struct BiasHullParams {
     const float* bias;
     int64_t bias_b, bias_h, bias_r;
-    int32_t* kv_start;         // out [B, Lq]
-    int32_t* kv_end;           // out [B, Lq]
+    int32_t* kv_start;         // [B, Lq]: written by the hull kernel, read by the interval test
+    int32_t* kv_end;           // [B, Lq]
     int B, heads, Lq, Lkv;     // heads: 1 (bias broadcast over heads) or Hq
+    int32_t* flag;             // interval test only: set to 1 when the bias is not 0 everywhere inside the hull
 };
 hipError_t launch_bias_hull(const BiasHullParams& p, hipStream_t st);
+hipError_t launch_bias_interval(const BiasHullParams& p, hipStream_t st);
 
 struct PreParams {
     const uint16_t* o;

@@ -256,6 +256,27 @@ __global__ __launch_bounds__(256) void bias_hull_kernel(const BiasHullParams p) 
     }
 }
 
+// One wave per (b, text row): sets *p.flag when an entry of the row's bias inside [kv_start, kv_end)
+// is not exactly zero, i.e. when the bias is more than the interval mask its hull describes.
+__global__ __launch_bounds__(256) void bias_interval_kernel(const BiasHullParams p) {
+    const int64_t rw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (rw >= (int64_t)p.B * p.Lq) return;
+    const int b = (int)(rw / p.Lq), row = (int)(rw % p.Lq);
+    const int lo = max(p.kv_start[rw], 0), hi = min(p.kv_end[rw], p.Lkv);
+    bool other = false;
+    for (int h = 0; h < p.heads; ++h) {
+        const float* br = p.bias + b * p.bias_b + h * p.bias_h + (int64_t)row * p.bias_r;
+        for (int k0 = (lo & ~3) + 4 * lane; k0 < hi; k0 += 256) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(br + k0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (k0 + j >= lo && k0 + j < hi && !(v[j] == 0.f)) other = true;
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64(other) != 0 && lane == 0) atomicOr(p.flag, 1);
+}
+
 // One wave per (group of row tiles, b): the hull of the rows' key intervals in whole token blocks.
 __global__ __launch_bounds__(64) void bwd_hull_kernel(const LiveParams p) {
     const int grp = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
@@ -450,6 +471,12 @@ hipError_t launch_bias_hull(const BiasHullParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.Lq;
     if (rows == 0) return hipSuccess;
     return launch1(bias_hull_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), st, p);
+}
+
+hipError_t launch_bias_interval(const BiasHullParams& p, hipStream_t st) {
+    const int64_t rows = (int64_t)p.B * p.Lq;
+    if (rows == 0) return hipSuccess;
+    return launch1(bias_interval_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), st, p);
 }
 
 hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {

@@ -49,6 +49,7 @@ SYMBOLS = {
     "lvx_noalloc_scratch_bytes": (C.c_size_t, []),
     "lvx_merge": (C.c_int, [_SHAPE, _T, _P, _T, _P, C.c_int32, C.c_int32, _P]),
     "lvx_bias_hull": (C.c_int, [_SHAPE, _P, _P, _P]),
+    "lvx_bias_is_interval": (C.c_int, [_SHAPE, _P, _P, _P, _P]),
     "lvx_bwd_preprocess": (C.c_int, [_SHAPE, _T, _T, _P, C.c_int32, C.c_int32, _P]),
     "lvx_bwd": (C.c_int, [_SHAPE, _T, _T, _T, _T, _P, _P, _T, _T, _T, C.c_int32, C.c_int32, C.c_int32,
                           _P, C.c_size_t, _P]),

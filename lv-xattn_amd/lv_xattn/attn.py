@@ -87,10 +87,39 @@ def _dense_bias(bias_func, local_bias_args, remote_bias_args, B, Hq, Lq, Lkv, de
     # rows are read with 16-byte loads: aligned base, strides multiples of 4, rows readable up to Lkv + pad
     strides_ok = all(bias.stride(i) % 4 == 0 or bias.shape[i] == 1 for i in range(3))
     if bias.stride(3) != 1 or bias.stride(2) < Lkv + pad or not strides_ok or bias.data_ptr() % 16:
+        kept = getattr(bias, "lvx_padded", None)
+        if kept is not None:
+            return kept
         padded = torch.zeros(*bias.shape[:3], Lkv + pad, dtype=torch.float32, device=dev)
         padded[..., :Lkv] = bias
-        bias = padded[..., :Lkv]
+        view = padded[..., :Lkv]
+        if getattr(bias, "lvx_reused", False):      # see _bias_and_hull: the copy is kept with it
+            view.lvx_reused = True
+            bias.lvx_padded = view
+        bias = view
     return bias
+
+
+def _bias_and_hull(bias: torch.Tensor, q, k):
+    """(bias or None, interval mask) for a dense bias given without a mask.  The mask is the hull of
+    what the bias leaves visible (ops.bias_hull), so the kernels skip what it masks anyway.  A bias
+    whose maker keeps it for later calls (attribute `lvx_reused`, set by the Hugging Face hook on
+    the mask it converts once per model call) is also tested once for being nothing but that
+    interval mask - 0 wherever it is not -inf - and is then dropped: the interval-mask kernels give
+    the same result without reading it.  The test waits for the GPU, which is why it is only made
+    for a bias that comes back; hull and verdict stay with the tensor (and so does the padded copy
+    _dense_bias may have to make of it), so a tensor marked `lvx_reused` must not be written to
+    afterwards."""
+    key = (tuple(q.shape[:3]), k.shape[2])
+    kept = getattr(bias, "lvx_hull", None)
+    if kept is not None and kept[0] == key:
+        return (None if kept[2] else bias), kept[1]
+    hull = ops.bias_hull(q, k, bias)
+    if not getattr(bias, "lvx_reused", False):
+        return bias, hull
+    exact = ops.bias_is_interval(q, k, bias, hull)
+    bias.lvx_hull = (key, hull, exact)
+    return (None if exact else bias), hull
 
 
 def auto_kv_splits(B: int, Hq: int, Hkv: int, rows: int, Lkv: int, target_wgs: int = 512) -> int:
@@ -136,7 +165,7 @@ def _attn_forward(q, k, v, causal, sm_scale, comm_mode, bias_func=None,
     if mask is not None:
         mask = mask.to(dev)
     elif bias is not None:
-        mask = ops.bias_hull(q_, k_, bias)    # skip what the bias masks out anyway
+        bias, mask = _bias_and_hull(bias, q_, k_)    # skip what the bias masks out anyway
 
     o = torch.empty(B, Hq, Lq, D, dtype=q_.dtype, device=dev)
     L = torch.empty(B * Hq, Lq, dtype=torch.float32, device=dev)
@@ -246,7 +275,7 @@ def _attn_backward(do, q, k, v, o, L, causal, sm_scale, comm_mode, backward_engi
     if mask is not None:
         mask = mask.to(dev)
     elif bias is not None:
-        mask = ops.bias_hull(q_, k_, bias)    # as in the forward: the same hull, hence the same pairs
+        bias, mask = _bias_and_hull(bias, q_, k_)    # as in the forward: the same hull, hence the same pairs
     L_ = L.to(torch.float32).reshape(B * Hq, Lq).contiguous()
 
     delta = workspace("bwd_delta", (B * Hq, Lq), torch.float32, dev)

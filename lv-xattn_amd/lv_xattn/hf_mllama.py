@@ -54,7 +54,9 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     row that sees every key.
     Where a row does see a key, its masked positions become -inf: the result is the same
     (exp(-30000) is already 0 there) and the kernels can then skip whole tiles outside the span
-    of the visible keys (ops.bias_hull), which is most of a Llama-3.2 mask."""
+    of the visible keys (ops.bias_hull), which is most of a Llama-3.2 mask.  A converted mask that
+    is kept is marked as such: the attention call then tests it once for being a pure interval
+    mask (every row sees one run of keys, bias 0 there) and, when it is, runs without the bias."""
     # an inference tensor (torch.inference_mode) has no version counter: its contents cannot be told
     # apart from an edited copy at the same address, so it is converted every time and not kept
     version = None if mask.is_inference() else mask._version
@@ -68,6 +70,7 @@ def _mask_bias(mask: torch.Tensor) -> torch.Tensor:
     # every cross-attention layer of a model gets the same mask, in forward and again in backward:
     # the last conversion is kept (with the mask itself, so that its address cannot be reused)
     if version is not None:
+        bias.lvx_reused = True      # attn._bias_and_hull: worth testing once whether it is an interval mask
         _bias_cache[:] = [key, bias, mask]
     return bias
 

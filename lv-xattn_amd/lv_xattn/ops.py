@@ -155,6 +155,18 @@ def bias_hull(q, k, bias: torch.Tensor) -> Mask:
     return Mask(None, start, end)
 
 
+def bias_is_interval(q, k, bias: torch.Tensor, hull: Mask) -> bool:
+    """Whether `bias` is nothing but the interval mask `hull` (from bias_hull): 0 wherever it is
+    not -inf.  fwd / bwd with `hull` alone then give what they give with the bias, through the
+    interval-mask kernels, which read no bias.  Waits for the GPU (one flag comes back)."""
+    s = _shape(q, k, 1.0, None, bias)
+    flag = torch.zeros(1, dtype=torch.int32, device=q.device)
+    rc = load().lvx_bias_is_interval(C.byref(s), hull.kv_start.data_ptr(), hull.kv_end.data_ptr(), flag.data_ptr(),
+                                     stream_ptr())
+    check(rc, "lvx_bias_is_interval")
+    return int(flag.item()) == 0
+
+
 def bwd_preprocess(o, dout, delta, row_begin=0, row_count=None) -> None:
     B, Hq, Lq, D = o.shape
     s = AttnShape(B, Hq, Hq, D, Lq, 1, dtype_code(o, dout), 1.0, None, None, None)

@@ -39,7 +39,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_version_and_error_strings(lib):
-    assert lib.lvx_version() == 101
+    assert lib.lvx_version() == 102
     assert lib.lvx_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert lib.lvx_strerror(code) not in (b"", b"unknown lvx error")
@@ -223,5 +223,5 @@ def test_plain_c_caller_compiles_against_the_header_and_calls_the_library(lib, t
     r = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     version, rc, msg, ws = r.stdout.strip().split("|")
-    assert int(version) == 101 and int(rc) == -4 and msg == "head_dim must be 128"
+    assert int(version) == 102 and int(rc) == -4 and msg == "head_dim must be 128"
     assert int(ws) == 4 * 8 * 64 * (128 * 2 + 4)

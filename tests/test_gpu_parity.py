@@ -643,6 +643,45 @@ def test_dense_bias_forward_backward(lvx, batched):
     assert dead.any() and (o.float().cpu()[dead] == 0).all() and (dq.float().cpu()[dead] == 0).all()
 
 
+@pytest.mark.parametrize("pure", [True, False])
+def test_a_kept_bias_that_is_an_interval_mask_runs_without_the_bias(lvx, monkeypatch, pure):
+    # what the Hugging Face hook hands over: the mask as a dense 0 / -inf bias that its maker keeps
+    # for every layer (marked lvx_reused).  Tested once for being nothing but per-row intervals, it is
+    # then dropped and the interval-mask kernels run; one finite entry inside a row's span keeps it.
+    from lv_xattn import ops
+    w = orc.make_inputs(orc.workload("cfg4s"))
+    t = w.tensors
+    allowed = orc.workload_allowed(w)                      # [B, Lq, Lkv] bool: an interval per row
+    bias = torch.zeros(w.B, 1, w.Lq, w.Lkv).masked_fill_(~allowed.view(w.B, 1, w.Lq, w.Lkv), float("-inf"))
+    if not pure:
+        b0, r0 = allowed.any(-1).nonzero()[0].tolist()
+        k0 = int(allowed[b0, r0].nonzero()[0])
+        bias[b0, 0, r0, k0] = 0.25
+    o_ref, l_ref = orc.round_loop_forward(t["q"], t["k"], t["v"], w.scale, w.rounds, bias=bias)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(t["do"], t["q"], t["k"], t["v"], o_ref, l_ref, w.scale,
+                                                    bias=bias, rounds=w.rounds)
+    bias_d = _dev(bias)
+    bias_d.lvx_reused = True
+    seen = {"fwd": [], "bwd": [], "hull": 0}
+    fwd0, bwd0, hull0 = ops.fwd, ops.bwd, ops.bias_hull
+    monkeypatch.setattr(ops, "fwd", lambda *a, **kw: (seen["fwd"].append(a[11] if len(a) > 11 else kw.get("bias")), fwd0(*a, **kw))[1])
+    monkeypatch.setattr(ops, "bwd", lambda *a, **kw: (seen["bwd"].append(kw.get("bias")), bwd0(*a, **kw))[1])
+    monkeypatch.setattr(ops, "bias_hull", lambda *a, **kw: (seen.__setitem__("hull", seen["hull"] + 1), hull0(*a, **kw))[1])
+    qd, kd, vd = _dev(t["q"]), _dev(t["k"]), _dev(t["v"])
+    for _ in range(2):      # the second pass finds hull and verdict with the tensor
+        _, _, _, o, L = lvx._attn_forward(qd, kd, vd, False, w.scale, None, lambda b: b, [bias_d], [], rounds=w.rounds)
+        dq, dk, dv = lvx._attn_backward(_dev(t["do"]), qd, kd, vd, o, L, False, w.scale, None, "flash", lambda b: b,
+                                        [bias_d], [], rounds=w.rounds)
+    torch.cuda.synchronize()
+    assert seen["hull"] == 1 and seen["fwd"] and seen["bwd"]
+    assert all((b is None) == pure for b in seen["fwd"] + seen["bwd"])
+    check_o(o, o_ref)
+    check_lse(L, l_ref)
+    check_grad(dq, dq_ref, "dQ")
+    check_grad(dk, dk_ref, "dK")
+    check_grad(dv, dv_ref, "dV")
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("per_head,per_sample", [(False, True), (True, True), (False, False)])
 def test_bias_hull_is_the_span_of_the_finite_entries(lvx, per_head, per_sample):
