@@ -62,6 +62,23 @@ def _fwd(lib, shape, q=None, k=None, v=None, o=None, lse=0x2000, rb=0, rc=64, sp
     return lib.lvx_fwd(C.byref(shape), C.byref(q), C.byref(k), C.byref(v), C.byref(o), lse, rb, rc, splits, ws, wsb, None)
 
 
+def test_the_build_entry_point_accepts_the_library_it_built(lib):
+    # build() of the driver's entry file ends with this check; it reads the version from the header
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("graft_entry", os.path.join(ROOT, "__graft_entry__.py"))
+    entry = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(entry)
+    entry.check_abi_version(lib)
+
+    class Stale:
+        @staticmethod
+        def lvx_version():
+            return lib.lvx_version() - 1
+
+    with pytest.raises(RuntimeError, match="ABI"):
+        entry.check_abi_version(Stale)
+
+
 def test_forward_rejects_bad_arguments_before_launch(lib):
     assert _fwd(lib, _shape(D=64)) == -4
     assert _fwd(lib, _shape(dtype=3)) == -5            # 1 = bf16, 2 = fp16
