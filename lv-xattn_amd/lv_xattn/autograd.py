@@ -84,7 +84,9 @@ def create_attention_class(attention_mode: str = "lv_xattn", no_overlap: bool = 
     k_norm_eps=1e-5, bias_func=None, *bias_args) -> o: q given, K/V recomputed:
 
     Forward: K, V = kv_proj(x_vis); o, L = attention; saves (q, x_vis, w_k, w_v,
-    o, L) - K and V are dropped.  Backward: recomputes K, V by the same GEMMs,
+    o, L) - K and V are dropped.  (q stays: [B, Hq, Lq, D], 32 MiB at B1 Hq32 Lq4096, which is
+    more than the 25 MiB of K and V at Lkv 6404 that are not kept; the run_function form above
+    saves the layer input instead and recomputes q as well.)  Backward: recomputes K, V by the same GEMMs,
     runs the attention backward, then dX_vis = dK W_k^T + dV W_v^T (and, with
     `weight_grads`, dW_k = X^T dK, dW_v = X^T dV).  With `k_norm_weight` K is
     RMS-normalised per head in the projection's epilogue (the k_norm of
