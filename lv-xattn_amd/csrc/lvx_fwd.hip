@@ -6,6 +6,8 @@
 // ONE q head; the 4 waves of a group cover the q heads that share a kv head
 // (G = 4: four heads x 32 rows; G = 1: one head x 128 rows), so the K/V tile
 // staged in LDS is read by the whole GQA group and nothing is expanded in HBM.
+// (The bf16 kernel without a dense bias, fwd_kernel_pipe, also has a wide form in which
+// a wavefront owns 64 rows; see there.)
 //
 // Per 64-key tile and wave (all MFMA are v_mfma_f32_32x32x16_bf16):
 //   S^T[key, row]  = K_tile (A, from LDS)  x  Q^T (B, 32 VGPRs held for the whole kernel)
@@ -502,9 +504,7 @@ __global__ __launch_bounds__(256, 3 - NBLK) void fwd_kernel_pipe(const FwdParams
     if (krow_b == vrow_b) {
         const int fa = max(t_begin, (in_lo + BN - 1) / BN);
         const int fb = min(t_end, min(in_hi, kv_hi) / BN);
-#ifndef LVX_FWD_NOFAST
         if (fb - fa >= 3) { ta = fa; n_fast = (fb - fa - 1) | 1; }
-#endif
     }
 
     for (int phase = 0; phase < 3; ++phase) {
