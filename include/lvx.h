@@ -91,11 +91,11 @@ const char* lvx_strerror(int code);
  * kv_splits > 1 cuts the shard into that many key ranges computed by separate
  * work-groups and folded before return; it needs a workspace of
  * lvx_fwd_workspace_bytes(shape, row_count, kv_splits) bytes.
- * The bf16 kernel without a dense bias has two forms: a wavefront owns 32 text rows, or
- * 64 rows and its SIMD to itself (half the LDS traffic per MFMA, one work-group per CU).
- * The second is picked when there is no interval mask, row_count is a whole number of
- * work-group row blocks and the launch has at least one work-group per CU; the
- * environment variable LVX_FWD_WIDE (0 / 1, read at every call) overrides the choice.
+ * The bf16 kernel without a dense bias or an interval mask has two forms: a wavefront owns
+ * 32 text rows, or 64 rows and its SIMD to itself (half the LDS traffic per MFMA, one
+ * work-group per CU).  The second is picked when row_count is a whole number of work-group
+ * row blocks and the launch has at least one work-group per CU; the environment variable
+ * LVX_FWD_WIDE (0 / 1, read at every call) overrides the choice.
  * Both forms give results within the same tolerance of each other, not the same bits.
  */
 int lvx_fwd(const lvx_attn_shape* shape, const lvx_tensor* q, const lvx_tensor* k,

@@ -127,8 +127,8 @@ static int cu_count();
 // CU): bf16 without a dense bias or an interval mask, whole 64-row blocks, and enough work-groups
 // that every CU has one.
 static bool fwd_wide(const lvx_attn_shape* s, int32_t row_count, int rs, int kv_splits) {
-    if (const char* e = getenv("LVX_FWD_WIDE")) return atoi(e) != 0 && s->dtype == LVX_BF16 && !s->bias;
     if (s->dtype != LVX_BF16 || s->bias || s->kv_start) return false;
+    if (const char* e = getenv("LVX_FWD_WIDE")) return atoi(e) != 0;
     if (row_count % (64 * rs) != 0) return false;
     const int64_t wgs = (int64_t)s->B * (s->Hq / (4 / rs)) * (row_count / (64 * rs)) * kv_splits;
     return wgs >= cu_count();

@@ -6,7 +6,7 @@
 // ONE q head; the 4 waves of a group cover the q heads that share a kv head
 // (G = 4: four heads x 32 rows; G = 1: one head x 128 rows), so the K/V tile
 // staged in LDS is read by the whole GQA group and nothing is expanded in HBM.
-// (The bf16 kernel without a dense bias, fwd_kernel_pipe, also has a wide form in which
+// (The bf16 kernel without a dense bias or an interval mask, fwd_kernel_pipe, also has a wide form in which
 // a wavefront owns 64 rows; see there.)
 //
 // Per 64-key tile and wave (all MFMA are v_mfma_f32_32x32x16_bf16):
@@ -331,19 +331,19 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 // the same for the wide loop (gen_fwd_loop_wide.py): its working VGPRs and the accumulation registers
 #define LVX_FWD_WIDE_CLOBBERS "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191"
 
-// The bf16 kernel without a dense bias (the one the benchmarks run): fwd_kernel's mapping, LDS
+// The bf16 kernel without a dense bias or an interval mask (the one the benchmarks run): fwd_kernel's mapping, LDS
 // layout and tile code, but the run of key tiles that every row of the work-group sees in full
 // goes through a hand-scheduled loop (gen_fwd_loop.py) in which every wave interleaves the
 // MFMAs of a tile with the exponentials of that tile and the scores of the next one.  The
-// tiles before and after that run (mask edges, the partial last tile) take the plain tile code.
+// tiles before and after that run (the partial last tile, rows past the window) take the plain tile code.
 //
 // NBLK = 2 is the wide form: a wave owns two blocks of 32 rows of its head (64 rows), has its
 // SIMD to itself (one work-group per CU, 512 registers per lane) and feeds every K / V operand it
 // reads from LDS to two MFMAs, one per block (gen_fwd_loop_wide.py): half the LDS reads and half
 // the global -> LDS bytes per MFMA.
-template <bool MASKED, int NBLK>
+template <int NBLK>
 __global__ __launch_bounds__(256, 3 - NBLK) void fwd_kernel_pipe(const FwdParams p) {
-    constexpr bool BIAS = false, F16 = false;
+    constexpr bool MASKED = false, BIAS = false, F16 = false;
     using E = Elt<F16>;
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
@@ -727,13 +727,11 @@ hipError_t launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
     if (p.bias) {
         if (masked) return launch1((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), st, p);
         else return launch1((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), st, p);
-    } else if (!F16) {
-        if (p.wide) {
-            if (masked) return launch1((fwd_kernel_pipe<true, 2>), dim3(grid), dim3(256), st, p);
-            else return launch1((fwd_kernel_pipe<false, 2>), dim3(grid), dim3(256), st, p);
-        }
-        if (masked) return launch1((fwd_kernel_pipe<true, 1>), dim3(grid), dim3(256), st, p);
-        else return launch1((fwd_kernel_pipe<false, 1>), dim3(grid), dim3(256), st, p);
+    } else if (!F16 && !masked) {
+        // (with an interval mask the plain kernel is the faster one: the edges of the rows' intervals leave
+        // the hand-scheduled loop short runs, and its register needs cost the tile code around it)
+        if (p.wide) return launch1((fwd_kernel_pipe<2>), dim3(grid), dim3(256), st, p);
+        return launch1((fwd_kernel_pipe<1>), dim3(grid), dim3(256), st, p);
     } else {
         if (masked) return launch1((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), st, p);
         else return launch1((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), st, p);

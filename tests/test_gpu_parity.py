@@ -267,10 +267,11 @@ def test_preprocess_delta(lvx):
 # ------------------------------------------------------------------ forward
 @pytest.fixture(params=["auto", "wide"])
 def form(request, monkeypatch):
-    """The forward kernel has two forms: a wave owns 32 rows, or 64 rows and its SIMD (picked for bf16
-    launches without mask or bias that give every CU a work-group).  'wide' forces the second on
-    these small shapes - also with masks, ragged row counts and key splits - through the
-    environment variable the library reads at every call."""
+    """The bf16 forward kernel for launches without interval mask or bias has two forms: a wave owns 32
+    rows, or 64 rows and its SIMD (picked when every CU gets a work-group).  'wide' forces the second
+    on these small shapes - also with ragged row counts, ragged key lengths, key splits and incoming
+    accumulators - through the environment variable the library reads at every call (masked launches
+    take the plain kernel either way)."""
     if request.param == "wide":
         monkeypatch.setenv("LVX_FWD_WIDE", "1")
     return request.param
