@@ -71,6 +71,7 @@ static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 
 namespace {
 constexpr int MAX_DEVICES = 64;
+constexpr int MAX_RANKED_GROUPS = 1024;    // 256-row groups of a masked backward that are still ranked by length
 std::mutex scratch_mutex;
 void* scratch_ptr[MAX_DEVICES];      // per device: where that device keeps `scratch`
 
@@ -435,9 +436,9 @@ static int dq_k_splits(const lvx_attn_shape* s, int32_t row_count, int* split_le
 // Regions of the backward workspace, in order: dS^T tiles; fp32 dK/dV scratch (split-steps mode
 // with bf16 outputs); row metadata records (2 floats per row and head); fp32 dQ partial tiles,
 // one slice per split (split dQ contraction only); with an interval mask the live-tile tables (group hulls, runs
-// of live tiles per token block).  Every region is a multiple of 16 bytes.
+// of live tiles per token block, the groups ranked by hull length).  Every region is a multiple of 16 bytes.
 struct BwdWorkspace {
-    size_t ds, dkv, meta, dq32, hull, runs, total;
+    size_t ds, dkv, meta, dq32, hull, runs, order, total;
     int n_tiles, group, n_groups;
 };
 
@@ -461,6 +462,7 @@ static BwdWorkspace bwd_workspace(const lvx_attn_shape* s, int32_t row_count) {
         const size_t nkb = tokens / 128;
         w.hull = off; off += up16((size_t)s->B * w.n_groups * 2 * sizeof(int32_t));
         w.runs = off; off += (size_t)s->B * nkb * 8 * sizeof(int32_t);
+        w.order = off; off += up16((size_t)s->B * w.n_groups * sizeof(int32_t));
     }
     w.total = off;
     return w;
@@ -538,10 +540,14 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         p.meta = meta;
     }
     int32_t* hull = nullptr;
+    int32_t* order = nullptr;
     if (s->kv_start) {
         // interval mask: token blocks skip the row tiles that see none of their tokens
         hull = reinterpret_cast<int32_t*>(wsb + wsl.hull);
-        LiveParams lp{s->kv_len, s->kv_start, s->kv_end, hull, reinterpret_cast<int32_t*>(wsb + wsl.runs),
+        // the ranking is quadratic in the number of groups; where there are that many, the dQ
+        // GEMM's work-groups even out in index order
+        if (ks <= 1 && s->B * wsl.n_groups <= MAX_RANKED_GROUPS) order = reinterpret_cast<int32_t*>(wsb + wsl.order);
+        LiveParams lp{s->kv_len, s->kv_start, s->kv_end, hull, reinterpret_cast<int32_t*>(wsb + wsl.runs), order,
                       s->B, s->Lq, s->Lkv, row_begin,
                       row_begin + row_count, wsl.n_tiles, wsl.group, wsl.n_groups, p.n_kv_blocks};
         hipError_t el = launch_bwd_live(lp, st);
@@ -592,6 +598,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     g.k_len = s->kv_len;
     g.a_tiled_m = (int)(rows / 32);
     g.k_range = hull;            // [B][M tiles][2]: the group hulls are per M tile of this GEMM
+    g.m_order = order;
     fill_grid(g, row_count, s->D, 1, s->B * s->Hq);
     if (ks <= 1) return static_cast<int>(launch_gemm(g, true, true, st));
     // split contraction: every split stores its partial tiles in its own fp32 slice; the

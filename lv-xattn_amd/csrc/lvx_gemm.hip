@@ -115,20 +115,30 @@ __global__ __launch_bounds__(512, 1) void gemm_kernel(const GemmParams p) {
     constexpr int NRA = RA::NRD(WM), NRB = RB::NRD(WN);
     __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
 
-    const int wid0 = xcd_remap(blockIdx.x, p.total_wg);
+    const int wid0 = p.m_order ? (int)blockIdx.x : xcd_remap(blockIdx.x, p.total_wg);
     if (wid0 >= p.total_wg) return;
     const int nks = p.k_splits > 1 ? p.k_splits : 1;
     const int ksp = wid0 % nks;
     const int wid = wid0 / nks;
     const int tn = wid % p.tiles_n;
     const int t1 = wid / p.tiles_n;
-    const int tm = t1 % p.tiles_m;
-    const int t2 = t1 / p.tiles_m;
-    // the outer batch index (the sample, where there is one) varies fastest over the ids, so that
-    // every XCD's contiguous id range holds work of all samples (ragged ones differ in length)
-    const int zr = t2 % p.nbatch;
-    const int n_outer = p.nbatch / p.batch_inner;
-    const int z = (zr % n_outer) * p.batch_inner + zr / n_outer;
+    int tm, z, t2 = 0;
+    if (p.m_order) {
+        // M tiles with their own contraction ranges, ranked by length: the ids walk the ranking
+        // (the inner batch index fastest), so the hardware's in-order hand-out of work-groups
+        // starts the longest first, on every XCD alike
+        const int item = p.m_order[t1 / p.batch_inner];
+        tm = item % p.tiles_m;
+        z = (item / p.tiles_m) * p.batch_inner + t1 % p.batch_inner;
+    } else {
+        tm = t1 % p.tiles_m;
+        t2 = t1 / p.tiles_m;
+        // the outer batch index (the sample, where there is one) varies fastest over the ids, so that
+        // every XCD's contiguous id range holds work of all samples (ragged ones differ in length)
+        const int zr = t2 % p.nbatch;
+        const int n_outer = p.nbatch / p.batch_inner;
+        z = (zr % n_outer) * p.batch_inner + zr / n_outer;
+    }
     const GemmProblem& pr = p.prob[t2 / p.nbatch];
     const int m0 = tm * TM, n0 = tn * TN;
     const int zo = z / p.batch_inner, zi = z % p.batch_inner;
@@ -443,6 +453,7 @@ hipError_t launch_gemm(const GemmParams& p, bool a_mcontig, bool b_ncontig, hipS
         if (pr.nseg > 1 && (pr.lda[1] != pr.lda[0] || pr.ldb[1] != pr.ldb[0])) return hipErrorInvalidValue;
     }
     if (p.N > 128) return launch_cfg<2, 4, 4, 2, 4>(p, a_mcontig, b_ncontig, st);
+    if (p.m_order && (!p.k_range || p.nprob != 1 || p.k_splits > 1 || p.N > 128)) return hipErrorInvalidValue;
     if (p.M > 256 && !p.k_range) return launch_cfg<8, 1, 2, 4, 3>(p, a_mcontig, b_ncontig, st);
     return launch_cfg<4, 2, 2, 2, 4>(p, a_mcontig, b_ncontig, st);
 }

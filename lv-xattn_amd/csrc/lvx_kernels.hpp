@@ -129,6 +129,8 @@ struct LiveParams {
     int32_t* hull;             // out: [B][n_groups][2] token range (multiples of 128), (0, 0) if empty
     int32_t* live_runs;        // out, see BwdParams; a fifth run and later ones are merged into the
                                // fourth together with the gaps between them (visiting more is harmless)
+    int32_t* order;            // out (may be null): the B * n_groups group indices b * n_groups + grp,
+                               // longest hull first (ties in index order)
     int B, Lq, Lkv, row_begin, row_end, n_tiles, group, n_groups, n_kv_blocks;
 };
 hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st);
@@ -197,6 +199,10 @@ struct GemmParams {
     // Per (outer batch index, M tile) contraction range of segment 0: k_range[(zo * tiles_m +
     // tm) * 2 + {0, 1}] = first and one-past-last k (multiples of 128); null: all of K[0].
     const int32_t* k_range;
+    // With k_range (one problem, no split contraction): the (outer batch index, M tile) pairs
+    // zo * tiles_m + tm in the order the work-groups are to take them, longest range first
+    // (null: in index order).
+    const int32_t* m_order;
     int f16;                   // element type of A, B, C (and the norm weight): 0 bf16, 1 fp16
     // Split contraction (single-segment problems): k_splits work-groups per C tile, each
     // contracting k_split_len values of k (a multiple of 128) and storing its partial tile

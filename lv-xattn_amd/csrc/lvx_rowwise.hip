@@ -302,7 +302,22 @@ __global__ __launch_bounds__(64) void bwd_hull_kernel(const LiveParams p) {
 }
 
 // One thread per (token block, b): the runs of consecutive row tiles whose group's hull holds the block.
+// Blocks past those (b == 0 only) rank the groups by hull length, one thread per group.
 __global__ __launch_bounds__(64) void bwd_live_kernel(const LiveParams p) {
+    const int live_blocks = (p.n_kv_blocks + 63) / 64;
+    if ((int)blockIdx.x >= live_blocks) {
+        const int n = p.B * p.n_groups;
+        const int i = ((int)blockIdx.x - live_blocks) * 64 + threadIdx.x;
+        if (blockIdx.y != 0 || i >= n) return;
+        const int len = p.hull[2 * i + 1] - p.hull[2 * i];
+        int rank = 0;
+        for (int j = 0; j < n; ++j) {
+            const int lj = p.hull[2 * j + 1] - p.hull[2 * j];
+            rank += (lj > len || (lj == len && j < i)) ? 1 : 0;
+        }
+        p.order[rank] = i;
+        return;
+    }
     const int kblk = blockIdx.x * 64 + threadIdx.x, b = blockIdx.y;
     if (kblk >= p.n_kv_blocks) return;
     const int kvb = kblk * 128;
@@ -464,7 +479,8 @@ hipError_t launch_bwd_live(const LiveParams& p, hipStream_t st) {
     if (p.B <= 0 || p.n_groups <= 0 || p.n_kv_blocks <= 0) return hipSuccess;
     const hipError_t e = launch1(bwd_hull_kernel, dim3(p.n_groups, p.B), dim3(64), st, p);
     if (e != hipSuccess) return e;
-    return launch1(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64, p.B), dim3(64), st, p);
+    const int rank_blocks = p.order ? (p.B * p.n_groups + 63) / 64 : 0;
+    return launch1(bwd_live_kernel, dim3((p.n_kv_blocks + 63) / 64 + rank_blocks, p.B), dim3(64), st, p);
 }
 
 hipError_t launch_bias_hull(const BiasHullParams& p, hipStream_t st) {

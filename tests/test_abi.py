@@ -151,7 +151,7 @@ def test_other_entry_points_reject_bad_arguments(lib):
     # an interval mask adds the live-tile tables: one hull (2 ints, padded to 16 bytes) for the
     # single 256-row group and 8 ints per token block
     sm = _shape(kv_start=0x3000, kv_end=0x3100)
-    assert lib.lvx_bwd_workspace_bytes(C.byref(sm), 64) == need + 16 + 2 * 8 * 4
+    assert lib.lvx_bwd_workspace_bytes(C.byref(sm), 64) == need + 16 + 2 * 8 * 4 + 16
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need - 1, None) == -7
     assert lib.lvx_bwd(C.byref(s), C.byref(t), C.byref(t), C.byref(t), C.byref(t), 0x2000, 0x2000, C.byref(t),
