@@ -25,7 +25,7 @@ int check_tensor(const lvx_tensor* t) {
 int check_shape(const lvx_attn_shape* s) {
     if (!s) return LVX_ERR_NULL;
     if (s->dtype != LVX_BF16 && s->dtype != LVX_F16) return LVX_ERR_DTYPE;
-    if (s->D != 128) return LVX_ERR_HEAD_DIM;
+    if (s->D != 128 && s->D != 64) return LVX_ERR_HEAD_DIM;
     if (s->B <= 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Lq <= 0 || s->Lkv <= 0) return LVX_ERR_SHAPE;
     if (s->Hq % s->Hkv) return LVX_ERR_SHAPE;
     if (!(s->scale > 0.f) || !std::isfinite(s->scale)) return LVX_ERR_SCALE;
@@ -105,7 +105,7 @@ const char* lvx_strerror(int code) {
         case LVX_ERR_NULL: return "a required pointer is NULL";
         case LVX_ERR_ALIGN: return "pointer not 16-byte aligned or stride not a multiple of 8 elements";
         case LVX_ERR_SHAPE: return "bad sizes or row window";
-        case LVX_ERR_HEAD_DIM: return "head_dim must be 128";
+        case LVX_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
         case LVX_ERR_DTYPE: return "dtype must be LVX_BF16 or LVX_F16";
         case LVX_ERR_SCALE: return "scale must be finite and > 0";
         case LVX_ERR_WORKSPACE: return "workspace missing or too small";
@@ -125,10 +125,10 @@ size_t lvx_fwd_workspace_bytes(const lvx_attn_shape* s, int32_t row_count, int32
 static int cu_count();
 
 // Whether the forward runs in its wide form (a wave owns 64 rows and its SIMD; one work-group per
-// CU): bf16 without a dense bias or an interval mask, whole 64-row blocks, and enough work-groups
+// CU): bf16, head_dim 128, without a dense bias or an interval mask, whole 64-row blocks, and enough work-groups
 // that every CU has one.
 static bool fwd_wide(const lvx_attn_shape* s, int32_t row_count, int rs, int kv_splits) {
-    if (s->dtype != LVX_BF16 || s->bias || s->kv_start) return false;
+    if (s->dtype != LVX_BF16 || s->D != 128 || s->bias || s->kv_start) return false;
     if (const char* e = getenv("LVX_FWD_WIDE")) return atoi(e) != 0;
     if (row_count % (64 * rs) != 0) return false;
     const int64_t wgs = (int64_t)s->B * (s->Hq / (4 / rs)) * (row_count / (64 * rs)) * kv_splits;
@@ -153,6 +153,7 @@ static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tens
 
     FwdParams p{};
     p.f16 = s->dtype == LVX_F16;
+    p.D = s->D;
     p.q = static_cast<const uint16_t*>(q->ptr);
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
@@ -188,6 +189,7 @@ static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tens
         // merge is symmetric, so which side is "the accumulator" does not matter)
         MergeParams m{};
         m.f16 = s->dtype == LVX_F16;
+        m.D = s->D;
         m.o_acc = static_cast<uint16_t*>(o->ptr);
         m.l_acc = lse;
         m.o_part = static_cast<const uint16_t*>(o_in->ptr);
@@ -222,6 +224,7 @@ static int fwd_impl(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tens
 
     MergeParams m{};
     m.f16 = s->dtype == LVX_F16;
+    m.D = s->D;
     m.o_acc = static_cast<uint16_t*>(o->ptr);
     m.l_acc = lse;
     m.o_part = p.o;
@@ -307,6 +310,7 @@ int lvx_merge(const lvx_attn_shape* s, const lvx_tensor* o_acc, float* l_acc, co
     LVX_TRY(check_rows(s, row_begin, row_count));
     MergeParams m{};
     m.f16 = s->dtype == LVX_F16;
+    m.D = s->D;
     m.o_acc = static_cast<uint16_t*>(o_acc->ptr);
     m.l_acc = l_acc;
     m.o_part = static_cast<const uint16_t*>(o_part->ptr);
@@ -353,6 +357,7 @@ int lvx_bwd_preprocess(const lvx_attn_shape* s, const lvx_tensor* o, const lvx_t
     LVX_TRY(check_rows(s, row_begin, row_count));
     PreParams p{};
     p.f16 = s->dtype == LVX_F16;
+    p.D = s->D;
     p.o = static_cast<const uint16_t*>(o->ptr);
     p.dout = static_cast<const uint16_t*>(dout->ptr);
     p.delta = delta;
@@ -498,6 +503,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
 
     BwdParams p{};
     p.f16 = s->dtype == LVX_F16;
+    p.D = s->D;
     p.q = static_cast<const uint16_t*>(q->ptr);
     p.k = static_cast<const uint16_t*>(k->ptr);
     p.v = static_cast<const uint16_t*>(v->ptr);
@@ -571,6 +577,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
             // scratch memory order is [B, Lkv, Hkv, D]: cast with (H, L) = (Lkv, Hkv)
             CastParams cp{};
             cp.f16 = p.f16;
+            cp.D = s->D;
             cp.src = scratch + i * dkv_elems;
             cp.dst = static_cast<uint16_t*>(t->ptr);
             cp.ds = Strides3{t->stride_b, t->stride_s, t->stride_h};
@@ -610,6 +617,7 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     if (e != hipSuccess) return static_cast<int>(e);
     CastParams cq{};
     cq.f16 = p.f16;
+    cq.D = s->D;
     cq.src = dq32;
     cq.dst = static_cast<uint16_t*>(dq->ptr) + (int64_t)row_begin * dq->stride_s;
     cq.ds = st3(dq);
@@ -627,10 +635,11 @@ int lvx_cast_f32(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, 
     if (!src) return LVX_ERR_NULL;
     LVX_TRY(check_tensor(dst));
     if (!aligned16(src)) return LVX_ERR_ALIGN;
-    if (D != 128) return LVX_ERR_HEAD_DIM;
+    if (D != 128 && D != 64) return LVX_ERR_HEAD_DIM;
     if (B <= 0 || H <= 0 || L <= 0) return LVX_ERR_SHAPE;
     CastParams p{};
     p.f16 = dtype == LVX_F16;
+    p.D = D;
     p.src = src;
     p.dst = static_cast<uint16_t*>(dst->ptr);
     p.ds = st3(dst);

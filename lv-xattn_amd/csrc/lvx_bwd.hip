@@ -73,9 +73,15 @@ constexpr float LOG2E = 1.4426950408889634f;
 #define LVX_BWD_LOOP_CLOBBERS "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199"
 
 // BIAS: a dense fp32 bias joins the exponent, P = exp2(S*c + bias*log2e - LSE*log2e).
-template <bool MASKED, bool BIAS, bool F16>
+// DH: head dimension, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk permutation
+// whatever DH is: with 64 only the first 8 chunks of a row hold data (the lanes that would load
+// the others repeat a chunk of the same row into positions nobody reads), and the k-steps of
+// S / dP and the 32-wide blocks of dV^T / dK^T past DH do not exist.
+template <int DH, bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     using E = Elt<F16>;
+    static_assert(DH == 64 || DH == 128, "head dimension");
+    constexpr int NKK = DH / 16, NDT = DH / 32;
     __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
     // per-row metadata of a staged tile, one per tile buffer: 8 x 16 bytes each of
     // LSE*log2e, delta*scale, kv_start, kv_end
@@ -127,12 +133,12 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     if (n_iter == 0 && p.dkv_mode != 0) return;
 
     // ---- resident B operand: this wave's K rows (P-wave) or V rows (D-wave)
-    bf16x8 breg[8];
+    bf16x8 breg[8];     // [NKK .. 8) stay unused when DH < 128
     {
         const uint16_t* base = d_role ? p.v + b * p.vs.b + hk * p.vs.h + (int64_t)my_kv * p.vs.s
                                       : p.k + b * p.ks.b + hk * p.ks.h + (int64_t)my_kv * p.ks.s;
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) breg[kk] = as_bf16x8(ldg16(base + kk * 16 + g * 8, kv_valid));
+        for (int kk = 0; kk < 8; ++kk) breg[kk] = as_bf16x8(ldg16(base + (kk < NKK ? kk : 0) * 16 + g * 8, kv_valid));
     }
     // ---- resident accumulator: dV^T (P-wave) or dK^T (D-wave), [128 d][32 tokens]
     f32x16 acc[4];
@@ -147,8 +153,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // rows 8w..8w+7 of the Q tile and of the dO tile as two 1 KiB loads each (4 rows
     // per load); lane i fills position i & 15 of row 4 ch + (i >> 4), ch = 2w, 2w+1.
     const int ld_r = 8 * slice + (lane >> 4);          // first of the two rows, the other is 4 further
-    const uint32_t ld_c0 = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice) & 3))) * 16u;
-    const uint32_t ld_c1 = (uint32_t)((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice + 1) & 3))) * 16u;
+    const uint32_t ld_c0 = (uint32_t)(((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice) & 3))) & (DH / 8 - 1)) * 16u;
+    const uint32_t ld_c1 = (uint32_t)(((lane & 15) ^ (((lane >> 4) << 2) | ((2 * slice + 1) & 3))) & (DH / 8 - 1)) * 16u;
     const uint32_t qrow_b = (uint32_t)p.qs.s * 2u, dorow_b = (uint32_t)p.dos.s * 2u;   // bytes per text row
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t meta0 = (uint32_t)(uintptr_t)&meta_s4[0][0];
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         }
         if (s_live) {
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk)
+            for (int kk = 0; kk < NKK; ++kk)
                 qa[kk] = *reinterpret_cast<const bf16x8*>(qt + row_rd + ((uint32_t)(kk * 32) ^ row_h));
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -285,13 +291,13 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) s_new[v] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) s_new = E::mfma(qa[kk], breg[kk], s_new);
+            for (int kk = 0; kk < NKK; ++kk) s_new = E::mfma(qa[kk], breg[kk], s_new);
         }
         if (pv_live) {
             // dO^T operands: requested once the S operands are consumed; they land while
             // the exp2 phase runs in the shadow of the S MFMAs
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     da[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(dot + t_rd[dt][0] + j * 4096));
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             *reinterpret_cast<u32x4*>(pbuf + pb_off) = pu[0];
             *reinterpret_cast<u32x4*>(pbuf + pb_off + 64 * 8) = pu[1];
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const u32x4 a = {da[dt][j][0][0], da[dt][j][0][1], da[dt][j][1][0], da[dt][j][1][1]};
@@ -354,7 +360,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         bf16x8 da[8];
         if (pv_live) {
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk)
+            for (int kk = 0; kk < NKK; ++kk)
                 da[kk] = *reinterpret_cast<const bf16x8*>(dor + row_rd + ((uint32_t)(kk * 32) ^ row_h));
         }
         if (ds_live) {
@@ -367,12 +373,12 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) dp_new[v] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) dp_new = E::mfma(da[kk], breg[kk], dp_new);
+            for (int kk = 0; kk < NKK; ++kk) dp_new = E::mfma(da[kk], breg[kk], dp_new);
         }
         if (ds_live) {
             // Q^T operands: requested once the dO operands are consumed
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     qa[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(qt + t_rd[dt][0] + j * 4096));
@@ -400,7 +406,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 *reinterpret_cast<u32x2*>(dsp + 8 * vg) = w;
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const u32x4 a = {qa[dt][j][0][0], qa[dt][j][0][1], qa[dt][j][1][0], qa[dt][j][1][1]};
@@ -483,7 +489,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         // Steady state of the plain bf16 kernel: steps 3 .. 3 + 6 trips - 1 (every one of them with all
         // its parts alive and a tile to request) run in the hand-scheduled loops of gen_bwd_loop.py,
         // six steps a trip; the steps after them continue below as if they had run here.
-        if constexpr (!MASKED && !BIAS && !F16 && !decltype(tail_c)::value) {
+        if constexpr (DH == 128 && !MASKED && !BIAS && !F16 && !decltype(tail_c)::value) {
             int trips = uniform32((n_iter - 5) / 6);
             if (i == 3 && trips >= 1 && (p.row_end - p.row_begin) % BM == 0) {
                 const int steps = 6 * trips;
@@ -592,7 +598,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         if (n_iter > 0) {
             float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EPS);
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) ep[l32 * EPS + dt * 32 + acc_row(v, g)] = acc[dt][v];
             __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): this wave's LDS writes have landed
@@ -603,7 +609,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 if (token >= p.Lkv) break;
                 float* op = obase + (int64_t)token * os.s;
                 unsafeAtomicAdd(op + lane, ep[t * EPS + lane]);
-                unsafeAtomicAdd(op + 64 + lane, ep[t * EPS + 64 + lane]);
+                if (DH == 128) unsafeAtomicAdd(op + 64 + lane, ep[t * EPS + 64 + lane]);
             }
         }
     } else if (my_kv < p.Lkv) {
@@ -613,7 +619,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         if (p.dkv_mode == 1) {
             float* op = reinterpret_cast<float*>(optr) + off;
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
@@ -625,7 +631,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
         } else {
             uint16_t* op = reinterpret_cast<uint16_t*>(optr) + off;
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
@@ -641,22 +647,24 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 }  // namespace
 
 namespace {
-template <bool F16>
+template <int DH, bool F16>
 hipError_t launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) return launch1((bwd_kernel<true, true, F16>), dim3(grid), dim3(NT), st, p);
-        else return launch1((bwd_kernel<false, true, F16>), dim3(grid), dim3(NT), st, p);
+        if (masked) return launch1((bwd_kernel<DH, true, true, F16>), dim3(grid), dim3(NT), st, p);
+        else return launch1((bwd_kernel<DH, false, true, F16>), dim3(grid), dim3(NT), st, p);
     } else {
-        if (masked) return launch1((bwd_kernel<true, false, F16>), dim3(grid), dim3(NT), st, p);
-        else return launch1((bwd_kernel<false, false, F16>), dim3(grid), dim3(NT), st, p);
+        if (masked) return launch1((bwd_kernel<DH, true, false, F16>), dim3(grid), dim3(NT), st, p);
+        else return launch1((bwd_kernel<DH, false, false, F16>), dim3(grid), dim3(NT), st, p);
     }
 }
 }  // namespace
 
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
-    if (p.f16) return launch_bwd_t<true>(p, masked, st);
-    return launch_bwd_t<false>(p, masked, st);
+    if (p.D == 64) return p.f16 ? launch_bwd_t<64, true>(p, masked, st) : launch_bwd_t<64, false>(p, masked, st);
+    if (p.D != 128) return hipErrorInvalidValue;
+    if (p.f16) return launch_bwd_t<128, true>(p, masked, st);
+    return launch_bwd_t<128, false>(p, masked, st);
 }
 
 }  // namespace lvx

@@ -46,9 +46,15 @@ constexpr float LOG2E_F = 1.4426950408889634f, LN2_F = 0.6931471805599453f;
 
 // BIAS: a dense fp32 bias is added to scale * S before the softmax; the scores are
 // then carried in log2 units (S*c + bias*log2e) instead of raw.
-template <bool MASKED, bool BIAS, bool F16>
+// DH: head dimension, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk permutation
+// whatever DH is: with 64 only the first 8 chunks of a row hold data (the lanes that would load
+// the others repeat a chunk of the same row into positions nobody reads), and the k-steps of
+// S^T and the 32-wide blocks of O^T past DH do not exist.
+template <int DH, bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     using E = Elt<F16>;
+    static_assert(DH == 64 || DH == 128, "head dimension");
+    constexpr int NKK = DH / 16, NDT = DH / 32;
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
 
@@ -113,11 +119,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     in_hi = __builtin_amdgcn_readfirstlane(in_hi);
 
     // Q^T as B operand, resident for the whole kernel
-    bf16x8 qreg[8];
+    bf16x8 qreg[NKK];
     {
         const uint16_t* qp = p.q + b * p.qs.b + h * p.qs.h + (int64_t)row * p.qs.s + g * 8;
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) qreg[kk] = as_bf16x8(ldg16(qp + kk * 16, row_ok));
+        for (int kk = 0; kk < NKK; ++kk) qreg[kk] = as_bf16x8(ldg16(qp + kk * 16, row_ok));
     }
 
     const char* kbase = reinterpret_cast<const char*>(p.k + b * p.ks.b + hk * p.ks.h);
@@ -128,7 +134,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     // of the K tile and of the V tile; lane i fills position i & 15 of row i >> 4.
     const int wave_u = wave;
     const int ld_r = lane >> 4;
-    const uint32_t ld_c = (uint32_t)((lane & 15) ^ ((ld_r << 2) | wave_u)) * 16u;   // chunk this lane fetches
+    const uint32_t ld_c = (uint32_t)(((lane & 15) ^ ((ld_r << 2) | wave_u)) & (DH / 8 - 1)) * 16u;   // chunk this lane fetches
     const uint32_t lds0 = (uint32_t)(uintptr_t)&kv_lds[0][0][0];
     auto issue = [&](int kv0, int buf) {
         const char* kb = kbase + (int64_t)kv0 * krow_b;
@@ -159,9 +165,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         }
     }
 
-    f32x16 acc[4];
+    f32x16 acc[NDT];
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
@@ -190,9 +196,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         // S^T = K Q^T : rows = keys (two 32-key sub-tiles), cols = text rows.
         // All 16 K operands are requested before the first MFMA, so the LDS
         // latency is paid once per tile and not once per k-step.
-        bf16x8 ka[8][2];
+        bf16x8 ka[NKK][2];
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
+        for (int kk = 0; kk < NKK; ++kk) {
             const char* kp = Ks + k_rd + ((uint32_t)(kk * 32) ^ k_h);
             ka[kk][0] = *reinterpret_cast<const bf16x8*>(kp);
             ka[kk][1] = *reinterpret_cast<const bf16x8*>(kp + 32 * 256);
@@ -202,15 +208,15 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s0[v] = 0.f; s1[v] = 0.f; }
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
+        for (int kk = 0; kk < NKK; ++kk) {
             s0 = E::mfma(ka[kk][0], qreg[kk], s0);
             s1 = E::mfma(ka[kk][1], qreg[kk], s1);
         }
         __builtin_amdgcn_sched_barrier(0);
         // V^T operands of this tile: requested now, they land during the softmax
-        u32x2 va[4][4][2];
+        u32x2 va[NDT][4][2];
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 va[dt][j][0] = lds_read_tr16(reinterpret_cast<const uint16_t*>(Vs + v_rd[dt][0] + j * 4096));
@@ -288,7 +294,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {   // the running max moved for some row
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[dt][v] *= alpha;
         }
@@ -296,7 +302,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         // O^T += V^T P^T
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const u32x4 a = {va[dt][j][0][0], va[dt][j][0][1], va[dt][j][1][0], va[dt][j][1][1]};
@@ -310,7 +316,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     if (row_ok) {
         uint16_t* op = p.o + split * p.o_split_stride + b * p.os.b + h * p.os.h + (int64_t)row * p.os.s;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int vg = 0; vg < 4; ++vg) {
                 u32x2 w;
@@ -721,27 +727,29 @@ __global__ __launch_bounds__(256, 3 - NBLK) void fwd_kernel_pipe(const FwdParams
 }  // namespace
 
 namespace {
-template <bool F16>
+template <int DH, bool F16>
 hipError_t launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
     const int grid = ((p.total_wg + 7) / 8) * 8;
     if (p.bias) {
-        if (masked) return launch1((fwd_kernel<true, true, F16>), dim3(grid), dim3(256), st, p);
-        else return launch1((fwd_kernel<false, true, F16>), dim3(grid), dim3(256), st, p);
-    } else if (!F16 && !masked) {
+        if (masked) return launch1((fwd_kernel<DH, true, true, F16>), dim3(grid), dim3(256), st, p);
+        else return launch1((fwd_kernel<DH, false, true, F16>), dim3(grid), dim3(256), st, p);
+    } else if (DH == 128 && !F16 && !masked) {
         // (with an interval mask the plain kernel is the faster one: the edges of the rows' intervals leave
         // the hand-scheduled loop short runs, and its register needs cost the tile code around it)
         if (p.wide) return launch1((fwd_kernel_pipe<2>), dim3(grid), dim3(256), st, p);
         return launch1((fwd_kernel_pipe<1>), dim3(grid), dim3(256), st, p);
     } else {
-        if (masked) return launch1((fwd_kernel<true, false, F16>), dim3(grid), dim3(256), st, p);
-        else return launch1((fwd_kernel<false, false, F16>), dim3(grid), dim3(256), st, p);
+        if (masked) return launch1((fwd_kernel<DH, true, false, F16>), dim3(grid), dim3(256), st, p);
+        else return launch1((fwd_kernel<DH, false, false, F16>), dim3(grid), dim3(256), st, p);
     }
 }
 }  // namespace
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
-    if (p.f16) return launch_fwd_t<true>(p, masked, st);
-    return launch_fwd_t<false>(p, masked, st);
+    if (p.D == 64) return p.f16 ? launch_fwd_t<64, true>(p, masked, st) : launch_fwd_t<64, false>(p, masked, st);
+    if (p.D != 128) return hipErrorInvalidValue;
+    if (p.f16) return launch_fwd_t<128, true>(p, masked, st);
+    return launch_fwd_t<128, false>(p, masked, st);
 }
 
 }  // namespace lvx

@@ -1,8 +1,8 @@
 // The HBM-bound row-wise kernels of the path: the LSE rescale-merge, the
 // backward preprocess (delta = rowsum(O * dO)) and the final fp32 -> bf16
-// rounding of an accumulator.  head_dim is 128: a row is 16 lanes x 16 bytes,
+// rounding of an accumulator.  With head_dim 128 a row is 16 lanes x 16 bytes,
 // so a 256-thread group streams 16 rows per pass with fully coalesced 256-byte
-// row segments.
+// row segments; with head_dim 64 it is 8 lanes and 32 rows per pass.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -13,8 +13,10 @@ namespace lvx {
 
 namespace {
 
-constexpr int D = 128;
 constexpr int MAX_PARTS = 16;
+
+// log2 of the 16-byte chunks (lanes) per row
+__device__ __forceinline__ int chunk_shift(int head_dim) { return head_dim == 64 ? 3 : 4; }
 
 template <class E>
 __device__ __forceinline__ void unpack8(u32x4 u, float f[8]) {
@@ -31,8 +33,9 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
     using E = Elt<F16>;
     const int nrows = p.row_end - p.row_begin;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int chunk = (int)(idx & 15);
-    const int64_t r = idx >> 4;
+    const int sh = chunk_shift(p.D);
+    const int chunk = (int)(idx & ((1 << sh) - 1));
+    const int64_t r = idx >> sh;
     if (r >= (int64_t)p.B * p.Hq * nrows) return;
     const int row = p.row_begin + (int)(r % nrows);
     const int bh = (int)(r / nrows);
@@ -107,8 +110,9 @@ __global__ __launch_bounds__(256) void merge_pair_kernel(const MergeParams p) {
     const int64_t total = (int64_t)p.B * p.Hq * nrows;
     const int64_t half = (total + 1) / 2;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int chunk = (int)(idx & 15);
-    const int64_t r0 = idx >> 4;
+    const int sh = chunk_shift(p.D);
+    const int chunk = (int)(idx & ((1 << sh) - 1));
+    const int64_t r0 = idx >> sh;
     if (r0 >= half) return;
     int64_t rr[2] = {r0, r0 + half};
     const bool ok1 = rr[1] < total;
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(256) void merge_pair_kernel(const MergeParams p) {
     }
 }
 
-// delta = rowsum(O * dO): 16 lanes x 16 bytes per row and tensor, two rows per thread with all
+// delta = rowsum(O * dO): 16 (head_dim 64: 8) lanes x 16 bytes per row and tensor, two rows per thread with all
 // four loads issued before the first use.  516 bytes per (row, head).
 template <bool F16>
 __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
@@ -165,9 +169,10 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
     const int64_t total = (int64_t)p.B * p.Hq * nrows;
     const int64_t half = (total + 1) / 2;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int chunk = (int)(idx & 15);
-    const int64_t r0 = idx >> 4;
-    const bool ok0 = r0 < half;                         // whole 16-lane groups share the flags
+    const int sh = chunk_shift(p.D);
+    const int chunk = (int)(idx & ((1 << sh) - 1));
+    const int64_t r0 = idx >> sh;
+    const bool ok0 = r0 < half;                         // the lanes of a row share the flags
     const bool ok1 = ok0 && r0 + half < total;
     const int64_t rr[2] = {ok0 ? r0 : 0, ok1 ? r0 + half : 0};
     u32x4 uo[2], ud[2];
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
-        s += __shfl_xor(s, 8);
+        if (sh == 4) s += __shfl_xor(s, 8);
         s += __shfl_xor(s, 4);
         s += __shfl_xor(s, 2);
         s += __shfl_xor(s, 1);
@@ -342,13 +347,15 @@ template <bool F16>
 __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     using E = Elt<F16>;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int chunk = (int)(idx & 15);
-    const int64_t r = idx >> 4;
+    const int sh = chunk_shift(p.D);
+    const int Dh = 8 << sh;
+    const int chunk = (int)(idx & ((1 << sh) - 1));
+    const int64_t r = idx >> sh;
     if (r >= (int64_t)p.B * p.H * p.L) return;
     const int row = (int)(r % p.L);
     const int bh = (int)(r / p.L);
     const int b = bh / p.H, h = bh % p.H;
-    const f32x4* s = reinterpret_cast<const f32x4*>(p.src + r * D + chunk * 8);
+    const f32x4* s = reinterpret_cast<const f32x4*>(p.src + r * Dh + chunk * 8);
     const f32x4 a = s[0], c = s[1];
     u32x4 u;
     u[0] = E::pack(a[0], a[1]);
@@ -364,12 +371,14 @@ template <bool F16>
 __global__ __launch_bounds__(256) void cast_t_kernel(const CastParams p) {
     using E = Elt<F16>;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)p.B * p.H * p.L * 16) return;
+    const int sh = chunk_shift(p.D);
+    const int Dh = 8 << sh;
+    if (idx >= ((int64_t)p.B * p.H * p.L << sh)) return;
     const int row = (int)(idx % p.L);
-    const int chunk = (int)((idx / p.L) & 15);
-    const int bh = (int)(idx / ((int64_t)p.L * 16));
+    const int chunk = (int)((idx / p.L) & ((1 << sh) - 1));
+    const int bh = (int)(idx / ((int64_t)p.L << sh));
     const int b = bh / p.H, h = bh % p.H;
-    const float* s = p.src + ((int64_t)bh * D + chunk * 8) * p.L + row;
+    const float* s = p.src + ((int64_t)bh * Dh + chunk * 8) * p.L + row;
     float a[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) a[j] = s[(int64_t)j * p.L];

@@ -41,19 +41,21 @@ def _usable(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
-HEAD_DIM = 128          # the head dimension the kernels are built for
+HEAD_DIM = 128          # the largest head dimension the kernels are built for
+NATIVE_HEAD_DIMS = (64, 128)
 
 
 def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
-    """Smaller head dimensions run zero-padded to 128: the padded columns add
-    nothing to q k^T, and the padded columns of O, dQ, dK and dV come out zero
-    and are cut off again.  Exact, at the cost of the padded arithmetic."""
+    """Head dimensions 64 and 128 have kernels.  Others below 128 run
+    zero-padded to the next of the two: the padded columns add nothing to
+    q k^T, and the padded columns of O, dQ, dK and dV come out zero and are cut
+    off again.  Exact, at the cost of the padded arithmetic."""
     D = t.shape[-1]
-    if D == HEAD_DIM:
+    if D in NATIVE_HEAD_DIMS:
         return t
     if D > HEAD_DIM:
         raise ValueError(f"head_dim {D} exceeds {HEAD_DIM}")
-    out = t.new_zeros(*t.shape[:-1], HEAD_DIM)
+    out = t.new_zeros(*t.shape[:-1], min(d for d in NATIVE_HEAD_DIMS if d >= D))
     out[..., :D] = t
     return out
 

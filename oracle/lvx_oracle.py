@@ -317,6 +317,7 @@ def workload(name: str) -> Workload:
         "cfg1s": dict(B=1, Hq=8, Hkv=2, D=128, Lq=512, Lkv=1601, rounds=4),
         "cfg2s": dict(B=1, Hq=8, Hkv=2, D=128, Lq=512, Lkv=1601, rounds=4, Dm=512),
         "cfg3s": dict(B=1, Hq=8, Hkv=2, D=128, Lq=256, Lkv=4096, rounds=16, Dm=512),
+        "cfg2s_d64": dict(B=1, Hq=8, Hkv=2, D=64, Lq=512, Lkv=1601, rounds=4, Dm=512),   # cfg0's head_dim
         "cfg4s": dict(B=2, Hq=8, Hkv=2, D=128, Lq=375, Lkv=802, rounds=4,
                       q_len=[375, 222], kv_len=[802, 401], image_tokens=401),
     }

@@ -39,7 +39,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
 
 
 def test_version_and_error_strings(lib):
-    assert lib.lvx_version() == 102
+    assert lib.lvx_version() == 103
     assert lib.lvx_strerror(0) == b"ok"
     for code in range(-8, 0):
         assert lib.lvx_strerror(code) not in (b"", b"unknown lvx error")
@@ -80,7 +80,8 @@ def test_the_build_entry_point_accepts_the_library_it_built(lib):
 
 
 def test_forward_rejects_bad_arguments_before_launch(lib):
-    assert _fwd(lib, _shape(D=64)) == -4
+    assert _fwd(lib, _shape(D=96)) == -4               # 64 and 128 have kernels
+    assert _fwd(lib, _shape(D=256)) == -4
     assert _fwd(lib, _shape(dtype=3)) == -5            # 1 = bf16, 2 = fp16
     assert _fwd(lib, _shape(Hq=7)) == -3
     assert _fwd(lib, _shape(scale=0.0)) == -6
@@ -165,7 +166,7 @@ def test_other_entry_points_reject_bad_arguments(lib):
     assert lib.lvx_bwd(C.byref(big), C.byref(t), C.byref(t), C.byref(t), C.byref(wide), 0x2000, 0x2000, C.byref(t),
                        C.byref(t), C.byref(t), 0, 0, 64, 0x4000, need_big, None) == -8
     assert b"not supported" in lib.lvx_strerror(-8)
-    assert lib.lvx_cast_f32(0x1000, C.byref(t), 1, 8, 64, 64, 1, None) == -4
+    assert lib.lvx_cast_f32(0x1000, C.byref(t), 1, 8, 64, 96, 1, None) == -4
     assert lib.lvx_kv_proj(0x1000, 512, 0x2000, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 250, 1, None) == -3
     assert lib.lvx_kv_proj(0x1000, 512, None, 0x3000, 256, 1, 0x4000, 0x5000, 256, 100, 512, 256, 2, None) == -1
     assert lib.lvx_dx_vis(0x1000, 0x1100, 256, 0x2000, 0x3000, 250, 1, 0x4000, 512, 100, 512, 256, 1, None) == -2
@@ -213,9 +214,9 @@ int main(int argc, char** argv) {
     if (!version || !strerr || !fwd || !ws) return 3;
     lvx_attn_shape s;
     memset(&s, 0, sizeof s);
-    s.B = 1; s.Hq = 8; s.Hkv = 2; s.D = 64; s.Lq = 64; s.Lkv = 256; s.dtype = LVX_BF16; s.scale = 0.125f;
+    s.B = 1; s.Hq = 8; s.Hkv = 2; s.D = 96; s.Lq = 64; s.Lkv = 256; s.dtype = LVX_BF16; s.scale = 0.125f;
     lvx_tensor t = {(void*)0x1000, 8 * 64 * 128, 64 * 128, 128};
-    int rc = fwd(&s, &t, &t, &t, &t, (float*)0x2000, 0, 64, 1, NULL, 0, NULL);   /* rejected on the host: D != 128 */
+    int rc = fwd(&s, &t, &t, &t, &t, (float*)0x2000, 0, 64, 1, NULL, 0, NULL);   /* rejected on the host: D is neither 64 nor 128 */
     s.D = 128;
     printf("%d|%d|%s|%zu\n", version(), rc, strerr(rc), ws(&s, 64, 4));
     return 0;
@@ -240,5 +241,5 @@ def test_plain_c_caller_compiles_against_the_header_and_calls_the_library(lib, t
     r = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     version, rc, msg, ws = r.stdout.strip().split("|")
-    assert int(version) == 102 and int(rc) == -4 and msg == "head_dim must be 128"
+    assert int(version) == 103 and int(rc) == -4 and msg == "head_dim must be 64 or 128"
     assert int(ws) == 4 * 8 * 64 * (128 * 2 + 4)

@@ -464,10 +464,15 @@ def test_backward_in_row_chunks_under_a_small_workspace_cap(lvx):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("batched", [False, True])
-def test_cfg0_shape_head_dim_64_runs_zero_padded(lvx, batched, dtype):
+def test_cfg0_shape_head_dim_64_runs_natively(lvx, batched, dtype, monkeypatch):
     """The CPU-only fp32 workload (head_dim 64, 4 rounds of 32 rows, 4096 keys) at its own
-    shape, rounded to a 16-bit type: smaller head dimensions run zero-padded to 128 in the host
-    loops, outputs and gradients come back at 64 columns."""
+    shape, rounded to a 16-bit type: head_dim 64 has kernels of its own, so the operators get
+    the tensors as they are (64 columns, nothing padded)."""
+    from lv_xattn import ops
+    dims = []
+    real_fwd, real_bwd = ops.fwd, ops.bwd
+    monkeypatch.setattr(ops, "fwd", lambda q_, *a, **kw: (dims.append(q_.shape[-1]), real_fwd(q_, *a, **kw))[1])
+    monkeypatch.setattr(ops, "bwd", lambda q_, *a, **kw: (dims.append(q_.shape[-1]), real_bwd(q_, *a, **kw))[1])
     w = orc.make_inputs(orc.workload("cfg0"))
     assert w.D == 64 and abs(w.scale - 0.125) < 1e-12
     w.dtype = dtype
@@ -479,6 +484,7 @@ def test_cfg0_shape_head_dim_64_runs_zero_padded(lvx, batched, dtype):
     dq, dk, dv = lvx._attn_backward(do, q, k, v, o, L, False, w.scale, None, "flash",
                                     rounds=w.rounds, batched=batched)
     torch.cuda.synchronize()
+    assert dims and set(dims) == {64}
     assert o.shape == q.shape and o.is_contiguous() and o.dtype == dtype
     assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
     check_o(o, ref["o"])
@@ -489,7 +495,8 @@ def test_cfg0_shape_head_dim_64_runs_zero_padded(lvx, batched, dtype):
 
 
 def test_head_dim_80_with_incoming_accumulator(lvx):
-    """Any head dimension up to 128 pads; the incoming accumulator pads with it."""
+    """Head dimensions without kernels of their own pad to the next one that has (80 -> 128); the
+    incoming accumulator pads with it."""
     g = torch.Generator().manual_seed(31)
     B, Hq, Hkv, D, Lq, Lkv = 2, 4, 2, 80, 96, 700
     q, k, v = (torch.randn(B, h, l, D, generator=g).bfloat16() for h, l in ((Hq, Lq), (Hkv, Lkv), (Hkv, Lkv)))
@@ -540,7 +547,7 @@ def test_backward_is_repeatable_up_to_atomic_order(lvx):
 
 
 # ------------------------------------------------------------------ recompute layer
-@pytest.mark.parametrize("name", ["cfg2s", "cfg3s"])
+@pytest.mark.parametrize("name", ["cfg2s", "cfg3s", "cfg2s_d64"])
 def test_recompute_layer_autograd(lvx, name):
     w = orc.make_inputs(orc.workload(name))
     t = w.tensors

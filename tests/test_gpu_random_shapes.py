@@ -43,8 +43,7 @@ def _piecewise_intervals(rng, B, Lq, Lkv, kv_len):
 
 
 def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided, dtype=torch.bfloat16,
-              sigma=1.0):
-    D = 128
+              sigma=1.0, D=128):
     scale = rng.choice([D ** -0.5, 0.05, 0.2])
     if strided:      # [B, S, H, D] memory viewed as [B, H, S, D]
         q = (sigma * torch.randn(B, Lq, Hq, D, generator=g)).to(dtype).transpose(1, 2)
@@ -69,7 +68,7 @@ def _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, stri
             mask = lvx.Mask(kl, start, end)
         else:
             mask = lvx.Mask(kl)
-    what = (f"B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv} P{rounds} batched={batched} mask={mask_kind} strided={strided} "
+    what = (f"B{B} Hq{Hq} Hkv{Hkv} D{D} Lq{Lq} Lkv{Lkv} P{rounds} batched={batched} mask={mask_kind} strided={strided} "
             f"{dtype}")
     print(what, flush=True)
 
@@ -102,6 +101,33 @@ def test_random_shape_forward_backward(lvx, seed):
     batched = rng.random() < 0.5
     mask_kind = ["none", "kv_len", "intervals", "intervals"][seed % 4]
     _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, batched, mask_kind, rng, g, strided=seed % 3 == 0)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shape_head_dim_64(lvx, seed, monkeypatch):
+    # head_dim 64 has kernels of its own (the reference takes powers of two up to 128,
+    # lv_xattn/attn.py:306-311): nothing is padded on the way, every mask kind, both element
+    # types, both memory layouts, with and without key splits / row splits
+    from lv_xattn import attn as ac
+    seen = []
+    real = ac._pad_head_dim
+    monkeypatch.setattr(ac, "_pad_head_dim", lambda t: (seen.append(t.shape[-1]), real(t))[1])
+    rng = random.Random(7000 + seed)
+    g = torch.Generator().manual_seed(8000 + seed)
+    B = rng.choice([1, 2, 3])
+    Hq, Hkv = rng.choice([(4, 4), (4, 2), (8, 2), (8, 1), (6, 3), (2, 1)])
+    if seed % 4 == 3:        # few rows against many keys: key splits, split dQ contraction
+        Lq, Lkv = rng.randint(1, 120), rng.randint(1100, 2600)
+    elif seed % 4 == 2:      # many rows against few keys: the row splits of the backward
+        Lq, Lkv, B, Hq, Hkv = 2560, rng.randint(100, 256), 1, 2, 1
+    else:
+        Lq, Lkv = rng.randint(1, 700), rng.randint(2, 900)
+    rounds = rng.choice([1, 2, 3, 5])
+    mask_kind = ["none", "kv_len", "intervals"][seed % 3]
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, rng.random() < 0.5, mask_kind, rng, g, strided=seed % 3 == 0,
+              dtype=dtype, sigma=[1.0, 0.5][seed % 2], D=64)
+    assert seen and set(seen) == {64}
 
 
 @pytest.mark.parametrize("seed", range(4))
