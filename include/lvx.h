@@ -41,7 +41,7 @@ extern "C" {
 #define LVX_ERR_NULL (-1)        /* a required pointer is NULL */
 #define LVX_ERR_ALIGN (-2)       /* pointer not 16-byte aligned / stride not a multiple of 8 */
 #define LVX_ERR_SHAPE (-3)       /* non-positive or inconsistent sizes, bad row window */
-#define LVX_ERR_HEAD_DIM (-4)    /* head_dim other than 64 or 128 */
+#define LVX_ERR_HEAD_DIM (-4)    /* head_dim other than 16, 32, 64 or 128 */
 #define LVX_ERR_DTYPE (-5)       /* dtype other than LVX_BF16 / LVX_F16 */
 #define LVX_ERR_SCALE (-6)       /* scale must be finite and > 0 */
 #define LVX_ERR_WORKSPACE (-7)   /* workspace missing or too small */
@@ -53,8 +53,8 @@ extern "C" {
 /* Sizes shared by the attention entry points. */
 typedef struct lvx_attn_shape {
     int32_t B, Hq, Hkv;
-    int32_t D;               /* head_dim: 64 or 128 (the reference takes powers of two up to 128,
-                                lv_xattn/attn.py:306-311; smaller ones run zero-padded by the caller) */
+    int32_t D;               /* head_dim: 16, 32, 64 or 128, the values the reference names
+                                (lv_xattn/attn.py:310; its Triton blocks need a power of two) */
     int32_t Lq;              /* text rows per sample (padded length)        */
     int32_t Lkv;             /* visual tokens per sample (padded length)    */
     int32_t dtype;           /* LVX_BF16 or LVX_F16: element type of q, k, v, o, dout, dq (and bf16/fp16 dk, dv) */

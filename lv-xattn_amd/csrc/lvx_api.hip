@@ -25,7 +25,7 @@ int check_tensor(const lvx_tensor* t) {
 int check_shape(const lvx_attn_shape* s) {
     if (!s) return LVX_ERR_NULL;
     if (s->dtype != LVX_BF16 && s->dtype != LVX_F16) return LVX_ERR_DTYPE;
-    if (s->D != 128 && s->D != 64) return LVX_ERR_HEAD_DIM;
+    if (s->D != 128 && s->D != 64 && s->D != 32 && s->D != 16) return LVX_ERR_HEAD_DIM;
     if (s->B <= 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Lq <= 0 || s->Lkv <= 0) return LVX_ERR_SHAPE;
     if (s->Hq % s->Hkv) return LVX_ERR_SHAPE;
     if (!(s->scale > 0.f) || !std::isfinite(s->scale)) return LVX_ERR_SCALE;
@@ -105,7 +105,7 @@ const char* lvx_strerror(int code) {
         case LVX_ERR_NULL: return "a required pointer is NULL";
         case LVX_ERR_ALIGN: return "pointer not 16-byte aligned or stride not a multiple of 8 elements";
         case LVX_ERR_SHAPE: return "bad sizes or row window";
-        case LVX_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
+        case LVX_ERR_HEAD_DIM: return "head_dim must be 16, 32, 64 or 128";
         case LVX_ERR_DTYPE: return "dtype must be LVX_BF16 or LVX_F16";
         case LVX_ERR_SCALE: return "scale must be finite and > 0";
         case LVX_ERR_WORKSPACE: return "workspace missing or too small";
@@ -635,7 +635,7 @@ int lvx_cast_f32(const float* src, const lvx_tensor* dst, int32_t B, int32_t H, 
     if (!src) return LVX_ERR_NULL;
     LVX_TRY(check_tensor(dst));
     if (!aligned16(src)) return LVX_ERR_ALIGN;
-    if (D != 128 && D != 64) return LVX_ERR_HEAD_DIM;
+    if (D != 128 && D != 64 && D != 32 && D != 16) return LVX_ERR_HEAD_DIM;
     if (B <= 0 || H <= 0 || L <= 0) return LVX_ERR_SHAPE;
     CastParams p{};
     p.f16 = dtype == LVX_F16;

@@ -73,15 +73,16 @@ constexpr float LOG2E = 1.4426950408889634f;
 #define LVX_BWD_LOOP_CLOBBERS "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199"
 
 // BIAS: a dense fp32 bias joins the exponent, P = exp2(S*c + bias*log2e - LSE*log2e).
-// DH: head dimension, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk permutation
-// whatever DH is: with 64 only the first 8 chunks of a row hold data (the lanes that would load
-// the others repeat a chunk of the same row into positions nobody reads), and the k-steps of
-// S / dP and the 32-wide blocks of dV^T / dK^T past DH do not exist.
+// DH: head dimension, 16, 32, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk
+// permutation whatever DH is: below 128 only the first DH / 8 chunks of a row hold data (the
+// lanes that would load the others repeat a chunk of the same row), and the k-steps of S / dP
+// and the 32-wide blocks of dV^T / dK^T past DH do not exist.  With 16 the one block of dV^T /
+// dK^T is half real: its upper 16 rows are products with those repeated chunks, never stored.
 template <int DH, bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     using E = Elt<F16>;
-    static_assert(DH == 64 || DH == 128, "head dimension");
-    constexpr int NKK = DH / 16, NDT = DH / 32;
+    static_assert(DH == 16 || DH == 32 || DH == 64 || DH == 128, "head dimension");
+    constexpr int NKK = DH / 16, NDT = DH >= 32 ? DH / 32 : 1;
     __shared__ __attribute__((aligned(1024))) uint16_t smem[SMEM_ELEMS];
     // per-row metadata of a staged tile, one per tile buffer: 8 x 16 bytes each of
     // LSE*log2e, delta*scale, kv_start, kv_end
@@ -608,7 +609,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
                 const int token = kvb + 32 * slice + t;
                 if (token >= p.Lkv) break;
                 float* op = obase + (int64_t)token * os.s;
-                unsafeAtomicAdd(op + lane, ep[t * EPS + lane]);
+                if (DH >= 64 || lane < DH) unsafeAtomicAdd(op + lane, ep[t * EPS + lane]);
                 if (DH == 128) unsafeAtomicAdd(op + 64 + lane, ep[t * EPS + 64 + lane]);
             }
         }
@@ -623,6 +624,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
+                    if (d >= DH) continue;      // only with DH = 16
                     f32x4 a = *reinterpret_cast<f32x4*>(op + d);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) a[r] += acc[dt][4 * vg + r];
@@ -635,6 +637,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 #pragma unroll
                 for (int vg = 0; vg < 4; ++vg) {
                     const int d = dt * 32 + 8 * vg + 4 * g;
+                    if (d >= DH) continue;      // only with DH = 16
                     u32x2 a;
                     a[0] = E::pack(acc[dt][4 * vg], acc[dt][4 * vg + 1]);
                     a[1] = E::pack(acc[dt][4 * vg + 2], acc[dt][4 * vg + 3]);
@@ -661,10 +664,13 @@ hipError_t launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
 }  // namespace
 
 hipError_t launch_bwd(const BwdParams& p, bool masked, hipStream_t st) {
-    if (p.D == 64) return p.f16 ? launch_bwd_t<64, true>(p, masked, st) : launch_bwd_t<64, false>(p, masked, st);
-    if (p.D != 128) return hipErrorInvalidValue;
-    if (p.f16) return launch_bwd_t<128, true>(p, masked, st);
-    return launch_bwd_t<128, false>(p, masked, st);
+    switch (p.D) {
+        case 16: return p.f16 ? launch_bwd_t<16, true>(p, masked, st) : launch_bwd_t<16, false>(p, masked, st);
+        case 32: return p.f16 ? launch_bwd_t<32, true>(p, masked, st) : launch_bwd_t<32, false>(p, masked, st);
+        case 64: return p.f16 ? launch_bwd_t<64, true>(p, masked, st) : launch_bwd_t<64, false>(p, masked, st);
+        case 128: return p.f16 ? launch_bwd_t<128, true>(p, masked, st) : launch_bwd_t<128, false>(p, masked, st);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace lvx

@@ -46,15 +46,16 @@ constexpr float LOG2E_F = 1.4426950408889634f, LN2_F = 0.6931471805599453f;
 
 // BIAS: a dense fp32 bias is added to scale * S before the softmax; the scores are
 // then carried in log2 units (S*c + bias*log2e) instead of raw.
-// DH: head dimension, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk permutation
-// whatever DH is: with 64 only the first 8 chunks of a row hold data (the lanes that would load
-// the others repeat a chunk of the same row into positions nobody reads), and the k-steps of
-// S^T and the 32-wide blocks of O^T past DH do not exist.
+// DH: head dimension, 16, 32, 64 or 128.  The LDS tiles keep their 256-byte rows and chunk
+// permutation whatever DH is: below 128 only the first DH / 8 chunks of a row hold data (the
+// lanes that would load the others repeat a chunk of the same row), and the k-steps of S^T and
+// the 32-wide blocks of O^T past DH do not exist.  With 16 the one block of O^T is half real:
+// its upper 16 rows are products with those repeated chunks and are never stored.
 template <int DH, bool MASKED, bool BIAS, bool F16>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     using E = Elt<F16>;
-    static_assert(DH == 64 || DH == 128, "head dimension");
-    constexpr int NKK = DH / 16, NDT = DH / 32;
+    static_assert(DH == 16 || DH == 32 || DH == 64 || DH == 128, "head dimension");
+    constexpr int NKK = DH / 16, NDT = DH >= 32 ? DH / 32 : 1;
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][2][TILE_BYTES];   // [buffer][K, V]
     __shared__ int red[4][4];
 
@@ -319,6 +320,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int vg = 0; vg < 4; ++vg) {
+                if (dt * 32 + 8 * vg + 4 * g >= DH) continue;      // only with DH = 16
                 u32x2 w;
                 w[0] = E::pack(acc[dt][4 * vg] * inv, acc[dt][4 * vg + 1] * inv);
                 w[1] = E::pack(acc[dt][4 * vg + 2] * inv, acc[dt][4 * vg + 3] * inv);
@@ -746,10 +748,13 @@ hipError_t launch_fwd_t(const FwdParams& p, bool masked, hipStream_t st) {
 }  // namespace
 
 hipError_t launch_fwd(const FwdParams& p, bool masked, hipStream_t st) {
-    if (p.D == 64) return p.f16 ? launch_fwd_t<64, true>(p, masked, st) : launch_fwd_t<64, false>(p, masked, st);
-    if (p.D != 128) return hipErrorInvalidValue;
-    if (p.f16) return launch_fwd_t<128, true>(p, masked, st);
-    return launch_fwd_t<128, false>(p, masked, st);
+    switch (p.D) {
+        case 16: return p.f16 ? launch_fwd_t<16, true>(p, masked, st) : launch_fwd_t<16, false>(p, masked, st);
+        case 32: return p.f16 ? launch_fwd_t<32, true>(p, masked, st) : launch_fwd_t<32, false>(p, masked, st);
+        case 64: return p.f16 ? launch_fwd_t<64, true>(p, masked, st) : launch_fwd_t<64, false>(p, masked, st);
+        case 128: return p.f16 ? launch_fwd_t<128, true>(p, masked, st) : launch_fwd_t<128, false>(p, masked, st);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace lvx

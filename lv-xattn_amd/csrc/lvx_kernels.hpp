@@ -35,7 +35,7 @@ struct FwdParams {
     const float* bias;         // dense additive bias or nullptr; element strides below
     int64_t bias_b, bias_h, bias_r;
     int B, Hq, Hkv, Lq, Lkv;
-    int D;                     // head dimension: 64 or 128
+    int D;                     // head dimension: 16, 32, 64 or 128
     int G;                     // q heads per kv head
     int HG;                    // q heads a work-group covers (one per wave)
     int RS;                    // row sub-tiles a work-group covers per head
@@ -65,7 +65,7 @@ struct MergeParams {
     int64_t l_in_bh;
     int B, Hq, Lq, row_begin, row_end;
     int f16;
-    int D;                     // head dimension, 64 or 128 (0 reads as 128)
+    int D;                     // head dimension: 16, 32, 64 or 128 (0 reads as 128)
 };
 
 // Per text row the hull of the keys a dense bias leaves visible (entries other than -inf).
@@ -87,7 +87,7 @@ struct PreParams {
     Strides3 os, ds;
     int B, Hq, Lq, row_begin, row_end;
     int f16;
-    int D;                     // head dimension, 64 or 128 (0 reads as 128)
+    int D;                     // head dimension: 16, 32, 64 or 128 (0 reads as 128)
 };
 
 struct BwdParams {
@@ -108,7 +108,7 @@ struct BwdParams {
     const float* bias;         // dense additive bias or nullptr; element strides below
     int64_t bias_b, bias_h, bias_r;
     int B, Hq, Hkv, Lq, Lkv, G;
-    int D;                     // head dimension: 64 or 128
+    int D;                     // head dimension: 16, 32, 64 or 128
     int row_begin, row_end;
     int n_kv_blocks, total_wg;
     int q_splits;              // work-groups sharing one token block, each taking a range of steps
@@ -164,7 +164,7 @@ struct CastParams {
     int nsum;         // transposed only: the result is the sum of nsum such sources (0 or 1: one),
     int64_t sum_stride;   // sum_stride floats apart
     int f16;          // destination type: 0 bf16, 1 fp16
-    int D;            // head dimension, 64 or 128 (0 reads as 128)
+    int D;            // head dimension: 16, 32, 64 or 128 (0 reads as 128)
 };
 
 // One GEMM problem C[M,N] = sum over segments A_s[M,K_s] * B_s[K_s,N].

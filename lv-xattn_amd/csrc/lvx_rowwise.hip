@@ -2,7 +2,7 @@
 // backward preprocess (delta = rowsum(O * dO)) and the final fp32 -> bf16
 // rounding of an accumulator.  With head_dim 128 a row is 16 lanes x 16 bytes,
 // so a 256-thread group streams 16 rows per pass with fully coalesced 256-byte
-// row segments; with head_dim 64 it is 8 lanes and 32 rows per pass.
+// row segments; with head_dim 64 / 32 / 16 it is 8 / 4 / 2 lanes and 32 / 64 / 128 rows per pass.
 #include "lvx_common.hpp"
 #include "lvx_kernels.hpp"
 
@@ -16,7 +16,9 @@ namespace {
 constexpr int MAX_PARTS = 16;
 
 // log2 of the 16-byte chunks (lanes) per row
-__device__ __forceinline__ int chunk_shift(int head_dim) { return head_dim == 64 ? 3 : 4; }
+__device__ __forceinline__ int chunk_shift(int head_dim) {
+    return head_dim == 64 ? 3 : head_dim == 32 ? 2 : head_dim == 16 ? 1 : 4;
+}
 
 template <class E>
 __device__ __forceinline__ void unpack8(u32x4 u, float f[8]) {
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(256) void merge_pair_kernel(const MergeParams p) {
     }
 }
 
-// delta = rowsum(O * dO): 16 (head_dim 64: 8) lanes x 16 bytes per row and tensor, two rows per thread with all
+// delta = rowsum(O * dO): head_dim / 8 lanes x 16 bytes per row and tensor, two rows per thread with all
 // four loads issued before the first use.  516 bytes per (row, head).
 template <bool F16>
 __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
@@ -195,9 +197,9 @@ __global__ __launch_bounds__(256) void preprocess_kernel(const PreParams p) {
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) s = fmaf(fo[j], fd[j], s);
-        if (sh == 4) s += __shfl_xor(s, 8);
-        s += __shfl_xor(s, 4);
-        s += __shfl_xor(s, 2);
+        if (sh >= 4) s += __shfl_xor(s, 8);
+        if (sh >= 3) s += __shfl_xor(s, 4);
+        if (sh >= 2) s += __shfl_xor(s, 2);
         s += __shfl_xor(s, 1);
         if ((k ? ok1 : ok0) && chunk == 0) *out[k] = s;
     }

@@ -42,14 +42,15 @@ def _usable(t: torch.Tensor) -> torch.Tensor:
 
 
 HEAD_DIM = 128          # the largest head dimension the kernels are built for
-NATIVE_HEAD_DIMS = (64, 128)
+NATIVE_HEAD_DIMS = (16, 32, 64, 128)
 
 
 def _pad_head_dim(t: torch.Tensor) -> torch.Tensor:
-    """Head dimensions 64 and 128 have kernels.  Others below 128 run
-    zero-padded to the next of the two: the padded columns add nothing to
-    q k^T, and the padded columns of O, dQ, dK and dV come out zero and are cut
-    off again.  Exact, at the cost of the padded arithmetic."""
+    """Head dimensions 16, 32, 64 and 128 (the reference's, lv_xattn/attn.py:306-311)
+    have kernels.  Others below 128 run zero-padded to the next of them: the
+    padded columns add nothing to q k^T, and the padded columns of O, dQ, dK and
+    dV come out zero and are cut off again.  Exact, at the cost of the padded
+    arithmetic."""
     D = t.shape[-1]
     if D in NATIVE_HEAD_DIMS:
         return t

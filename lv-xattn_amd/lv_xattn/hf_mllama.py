@@ -17,7 +17,7 @@ reference's `create_attention_class_save_qkv`, test_llama3.py:125-178).
 The registry is model-wide, so the causal self-attention layers arrive here as
 well; they are not this operator and are passed on to transformers' own
 implementation.  A cross-attention call the kernels do not cover (not bf16 on
-the GPU, head_dim other than 64 or 128 (the patched layer forward: 128), dropout) raises.
+the GPU, head_dim other than 16, 32, 64 or 128 (the patched layer forward: 128), dropout) raises.
 
 `patch_cross_attention_forward(model)` goes one step further, like the
 reference's recompute variant (`create_attention_class`,
@@ -108,9 +108,9 @@ def lv_xattn_attention_forward(module, query, key, value, attention_mask: Option
 
 
 def _require_supported(query, key, dropout):
-    if not (query.is_cuda and query.dtype in (torch.bfloat16, torch.float16) and query.shape[-1] in (64, 128) and dropout == 0.0
+    if not (query.is_cuda and query.dtype in (torch.bfloat16, torch.float16) and query.shape[-1] in (16, 32, 64, 128) and dropout == 0.0
             and query.shape[1] % key.shape[1] == 0):
-        raise LvxError("lv_xattn cross-attention needs bf16 or fp16 tensors on the GPU, head_dim 64 or 128, no dropout and "
+        raise LvxError("lv_xattn cross-attention needs bf16 or fp16 tensors on the GPU, head_dim 16, 32, 64 or 128, no dropout and "
                        f"Hkv | Hq; got {query.dtype} on {query.device}, q {tuple(query.shape)}, "
                        f"k {tuple(key.shape)}, dropout {dropout}")
 

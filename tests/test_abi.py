@@ -80,7 +80,7 @@ def test_the_build_entry_point_accepts_the_library_it_built(lib):
 
 
 def test_forward_rejects_bad_arguments_before_launch(lib):
-    assert _fwd(lib, _shape(D=96)) == -4               # 64 and 128 have kernels
+    assert _fwd(lib, _shape(D=96)) == -4               # 16, 32, 64 and 128 have kernels
     assert _fwd(lib, _shape(D=256)) == -4
     assert _fwd(lib, _shape(dtype=3)) == -5            # 1 = bf16, 2 = fp16
     assert _fwd(lib, _shape(Hq=7)) == -3
@@ -216,7 +216,7 @@ int main(int argc, char** argv) {
     memset(&s, 0, sizeof s);
     s.B = 1; s.Hq = 8; s.Hkv = 2; s.D = 96; s.Lq = 64; s.Lkv = 256; s.dtype = LVX_BF16; s.scale = 0.125f;
     lvx_tensor t = {(void*)0x1000, 8 * 64 * 128, 64 * 128, 128};
-    int rc = fwd(&s, &t, &t, &t, &t, (float*)0x2000, 0, 64, 1, NULL, 0, NULL);   /* rejected on the host: D is neither 64 nor 128 */
+    int rc = fwd(&s, &t, &t, &t, &t, (float*)0x2000, 0, 64, 1, NULL, 0, NULL);   /* rejected on the host: D is none of 16, 32, 64, 128 */
     s.D = 128;
     printf("%d|%d|%s|%zu\n", version(), rc, strerr(rc), ws(&s, 64, 4));
     return 0;
@@ -241,5 +241,5 @@ def test_plain_c_caller_compiles_against_the_header_and_calls_the_library(lib, t
     r = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     version, rc, msg, ws = r.stdout.strip().split("|")
-    assert int(version) == 103 and int(rc) == -4 and msg == "head_dim must be 64 or 128"
+    assert int(version) == 103 and int(rc) == -4 and msg == "head_dim must be 16, 32, 64 or 128"
     assert int(ws) == 4 * 8 * 64 * (128 * 2 + 4)

@@ -104,16 +104,17 @@ def test_random_shape_forward_backward(lvx, seed):
 
 
 @pytest.mark.parametrize("seed", range(12))
-def test_random_shape_head_dim_64(lvx, seed, monkeypatch):
-    # head_dim 64 has kernels of its own (the reference takes powers of two up to 128,
-    # lv_xattn/attn.py:306-311): nothing is padded on the way, every mask kind, both element
-    # types, both memory layouts, with and without key splits / row splits
+@pytest.mark.parametrize("D", [16, 32, 64])
+def test_random_shape_small_head_dims(lvx, D, seed, monkeypatch):
+    # the reference's head dimensions below 128 (16, 32, 64; lv_xattn/attn.py:306-311) have
+    # kernels of their own: nothing is padded on the way, every mask kind, both element types,
+    # both memory layouts, with and without key splits / row splits
     from lv_xattn import attn as ac
     seen = []
     real = ac._pad_head_dim
     monkeypatch.setattr(ac, "_pad_head_dim", lambda t: (seen.append(t.shape[-1]), real(t))[1])
-    rng = random.Random(7000 + seed)
-    g = torch.Generator().manual_seed(8000 + seed)
+    rng = random.Random(7000 + 100 * D + seed)
+    g = torch.Generator().manual_seed(8000 + 100 * D + seed)
     B = rng.choice([1, 2, 3])
     Hq, Hkv = rng.choice([(4, 4), (4, 2), (8, 2), (8, 1), (6, 3), (2, 1)])
     if seed % 4 == 3:        # few rows against many keys: key splits, split dQ contraction
@@ -126,8 +127,8 @@ def test_random_shape_head_dim_64(lvx, seed, monkeypatch):
     mask_kind = ["none", "kv_len", "intervals"][seed % 3]
     dtype = [torch.bfloat16, torch.float16][seed % 2]
     _run_case(lvx, B, Hq, Hkv, Lq, Lkv, rounds, rng.random() < 0.5, mask_kind, rng, g, strided=seed % 3 == 0,
-              dtype=dtype, sigma=[1.0, 0.5][seed % 2], D=64)
-    assert seen and set(seen) == {64}
+              dtype=dtype, sigma=[1.0, 0.5][seed % 2], D=D)
+    assert seen and set(seen) == {D}
 
 
 @pytest.mark.parametrize("seed", range(4))
