@@ -208,3 +208,51 @@ def test_more_than_four_runs_of_live_row_groups(lvx, batched):
     check_grad(dq, dq_ref, "dQ")
     check_grad(dk, dk_ref, "dK")
     check_grad(dv, dv_ref, "dV")
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_row_groups_with_hulls_of_many_lengths(lvx, seed):
+    # 2 samples x 8 groups of 256 rows whose hulls span 0 to 8 token blocks, some of equal length:
+    # the masked dQ GEMM takes its M tiles longest hull first, and every tile must still be
+    # written exactly once.  dQ starts as NaN, so a tile the ranking dropped would show (rows
+    # that see nothing get zeros, written by tiles with an empty range).
+    from lv_xattn import ops
+    rng = random.Random(9000 + seed)
+    g = torch.Generator().manual_seed(9100 + seed)
+    B, Hq, Hkv, Lq, Lkv, D = 2, 4, 2, 2048, 1024, 128
+    dtype = torch.bfloat16
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, Lkv, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, Lkv, D, generator=g).to(dtype)
+    do = torch.randn(B, Hq, Lq, D, generator=g).to(dtype)
+    start = torch.zeros(B, Lq, dtype=torch.int32)
+    end = torch.zeros(B, Lq, dtype=torch.int32)
+    lengths = [0, 0, 1, 2, 2, 3, 5, 8] * B
+    rng.shuffle(lengths)
+    for i, n in enumerate(lengths):
+        b, grp = divmod(i, 8)
+        if n:
+            first = rng.randint(0, 8 - n)
+            s, e = first * 128 + rng.randint(0, 100), (first + n) * 128 - rng.randint(0, 27)
+            start[b, grp * 256:(grp + 1) * 256], end[b, grp * 256:(grp + 1) * 256] = s, e
+    allowed = orc.interval_mask(start, end, Lkv)
+    scale = D ** -0.5
+    o_ref, l_ref = orc.attention_dense(q, k, v, scale, allowed=allowed)
+    dq_ref, dk_ref, dv_ref = orc.attention_backward(do, q, k, v, o_ref.to(dtype), l_ref, scale, allowed=allowed)
+    mask = lvx.Mask(None, start, end).to(DEV)
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    _, _, _, o, L = lvx._attn_forward(qd, kd, vd, False, scale, None, rounds=1, mask=mask, batched=True)
+    delta = torch.empty(B * Hq, Lq, device=DEV)
+    ops.bwd_preprocess(o, dod, delta)
+    dq = torch.full_like(qd, float("nan"))
+    dk = torch.empty(B, Lkv, Hkv, D, dtype=dtype, device=DEV).transpose(1, 2)
+    dv = torch.empty(B, Lkv, Hkv, D, dtype=dtype, device=DEV).transpose(1, 2)
+    ops.bwd(qd, kd, vd, dod, L.reshape(B * Hq, Lq).float().contiguous(), delta, dq, dk, dv, scale, mask=mask)
+    torch.cuda.synchronize()
+    assert not torch.isnan(dq.float()).any(), "an M tile of the dQ GEMM was not written"
+    check_o(o, o_ref)
+    check_grad(dq, dq_ref, "dQ")
+    check_grad(dk, dk_ref, "dK")
+    check_grad(dv, dv_ref, "dV")
+    dead = torch.isinf(l_ref).reshape(B, Hq, Lq)
+    assert (dq.float().cpu()[dead] == 0).all()
