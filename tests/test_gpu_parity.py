@@ -610,12 +610,13 @@ def test_save_qkv_autograd_wrapper(lvx):
 
 
 # ------------------------------------------------------------------ dense additive bias
+@pytest.mark.parametrize("name", ["cfg2s", "cfg2s_d64"])
 @pytest.mark.parametrize("batched", [False, True])
-def test_dense_bias_forward_backward(lvx, batched):
+def test_dense_bias_forward_backward(lvx, batched, name):
     # the reference's bias_func path (lv_xattn/attn.py:386-389, 504-507): bias [B,1,Lq,Lkv]
     # added after the scale; here with a Llama-style -inf pattern plus finite noise, a row
-    # that sees nothing, and a key length that is not a multiple of the tile
-    w = orc.make_inputs(orc.workload("cfg2s"))
+    # that sees nothing, and a key length that is not a multiple of the tile; at head_dim 128 and 64
+    w = orc.make_inputs(orc.workload(name))
     t = w.tensors
     B, Hq, Lq, Lkv = w.B, w.Hq, w.Lq, w.Lkv
     g = torch.Generator().manual_seed(77)
