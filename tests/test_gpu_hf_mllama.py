@@ -10,26 +10,28 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _layer(impl, dtype=torch.bfloat16):
+def _layer(impl, dtype=torch.bfloat16, hidden=1024):
     from transformers.models.mllama import modeling_mllama as m
     from transformers.models.mllama.configuration_mllama import MllamaTextConfig
-    cfg = MllamaTextConfig(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, num_hidden_layers=2,
+    cfg = MllamaTextConfig(hidden_size=hidden, num_attention_heads=8, num_key_value_heads=2, num_hidden_layers=2,
                            intermediate_size=256, cross_attention_layers=[1], vocab_size=128,
                            bos_token_id=1, eos_token_id=2, pad_token_id=0)
     cfg._attn_implementation = impl
     torch.manual_seed(3)
     layer = m.MllamaTextCrossAttention(cfg, layer_idx=1)
     with torch.no_grad():          # norm weights other than the all-ones initialisation
-        layer.q_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
-        layer.k_norm.weight.copy_(1.0 + 0.3 * torch.randn(128))
+        layer.q_norm.weight.copy_(1.0 + 0.3 * torch.randn(hidden // 8))
+        layer.k_norm.weight.copy_(1.0 + 0.3 * torch.randn(hidden // 8))
     return layer.to(device=DEV, dtype=dtype)
 
 
-@pytest.mark.parametrize("variant,dtype", [("interface", torch.bfloat16), ("recompute", torch.bfloat16),
-                                           ("recompute_intervals", torch.bfloat16),
-                                           ("interface", torch.float16), ("recompute", torch.float16)])
-def test_mllama_cross_attention_layer_matches_eager(variant, dtype):
-    """interface: the attention-interface hook (K/V kept for backward);
+@pytest.mark.parametrize("variant,dtype,hidden", [("interface", torch.bfloat16, 1024), ("recompute", torch.bfloat16, 1024),
+                                                  ("recompute_intervals", torch.bfloat16, 1024),
+                                                  ("interface", torch.float16, 1024), ("recompute", torch.float16, 1024),
+                                                  ("interface", torch.bfloat16, 512)])
+def test_mllama_cross_attention_layer_matches_eager(variant, dtype, hidden):
+    """interface: the attention-interface hook (K/V kept for backward), also with heads of 64
+    (hidden size 512);
     recompute: the patched forward (K/V + k_norm recomputed by the fused GEMM),
     with the dense mask or with the same mask as per-row key intervals."""
     pytest.importorskip("transformers")
@@ -37,17 +39,17 @@ def test_mllama_cross_attention_layer_matches_eager(variant, dtype):
     from lv_xattn import _lib, hf_mllama
     _lib.load()
     name = hf_mllama.register()
-    ref, new = _layer("eager", dtype), _layer(name, dtype)
+    ref, new = _layer("eager", dtype, hidden), _layer(name, dtype, hidden)
     new.load_state_dict(ref.state_dict())
-    assert ref.head_dim == 128
+    assert ref.head_dim == hidden // 8
     if variant != "interface":
         assert hf_mllama.patch_cross_attention_forward(new) == 1
 
     g = torch.Generator().manual_seed(11)
     B, Lq, Lkv = 2, 200, 1601
-    x = torch.randn(B, Lq, 1024, generator=g).to(dtype).to(DEV)
-    vis = torch.randn(B, Lkv, 1024, generator=g).to(dtype).to(DEV)
-    go = torch.randn(B, Lq, 1024, generator=g).to(dtype).to(DEV)
+    x = torch.randn(B, Lq, hidden, generator=g).to(dtype).to(DEV)
+    vis = torch.randn(B, Lkv, hidden, generator=g).to(dtype).to(DEV)
+    go = torch.randn(B, Lq, hidden, generator=g).to(dtype).to(DEV)
     # Llama-3.2 style additive mask: rows before the image see nothing (all entries
     # at the dtype minimum, as transformers builds it), sample 1 sees only the first tile
     neg = torch.finfo(dtype).min
