@@ -337,6 +337,35 @@ epilogue:
         }
         return;
     }
+    // A lane holds 4 consecutive columns of one C row, so storing from the registers writes 8
+    // bytes per lane into 32 different rows per instruction.  Where the tile fits the stage
+    // buffers (free by now) it goes through LDS instead and leaves as whole 512-byte row
+    // segments, 16 bytes per lane.  16-byte chunk c of row r sits at position c ^ (r & 31): the
+    // 32 rows one write instruction touches land in 32 different chunks, and a read instruction
+    // takes the 32 chunks of two rows - both conflict-free.  `pair(mt, nt, vg)`: the 4 values of
+    // accumulator tile (nt, mt), register group vg, as two packed words.
+    constexpr bool VIA_LDS = TN == 256 && TM * TN * 2 <= NS * STAGE;
+    auto store_via_lds = [&](auto pair, uint16_t* dst) __attribute__((always_inline)) {
+        __syncthreads();                    // every wave is done with what the buffers held
+#pragma unroll
+        for (int mt = 0; mt < WM; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < WN; ++nt)
+#pragma unroll
+                for (int vg = 0; vg < 4; ++vg) {
+                    const int ml = 32 * (WM * wm + mt) + l32;
+                    const int c = 4 * (WN * wn + nt) + vg;
+                    *reinterpret_cast<u32x2*>(lds + ml * (TN * 2) + ((c ^ l32) << 4) + g * 8) = pair(mt, nt, vg);
+                }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TM / 16; ++i) {
+            const int row = i * 16 + (tid >> 5), cc = tid & 31;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(lds + row * (TN * 2) + ((cc ^ (row & 31)) << 4));
+            const int m = m0 + row, n = n0 + cc * 8;
+            if (m < p.M && n < p.N) *reinterpret_cast<u32x4*>(dst + (int64_t)m * pr.ldc + n) = val;
+        }
+    };
     if (p.norm_w && t2 / p.nbatch == 0) {
         // RMS norm over each 128-column group (N and the tile are multiples of 128): the
         // group's columns sit in HW = 4 / WN waves with consecutive wn; row sums of squares
@@ -367,6 +396,35 @@ epilogue:
             for (int mt = 0; mt < WM; ++mt) rs[mt] += red[(pw * WM + mt) * 32 + l32];
         }
         const int groups = p.N >> 7;
+        if (VIA_LDS) {       // (N is a multiple of 128 here)
+            float rr[WM];
+#pragma unroll
+            for (int mt = 0; mt < WM; ++mt) {
+                const int m = m0 + 32 * (WM * wm + mt) + l32;
+                rr[mt] = rsqrtf(rs[mt] * (1.f / 128.f) + p.norm_eps);
+                const int ncol = n0 + 32 * WN * wn;
+                if (m < p.M && p.rstd && g == 0 && (wn & (HW - 1)) == 0 && ncol < p.N) p.rstd[(int64_t)m * groups + (ncol >> 7)] = rr[mt];
+            }
+            if (p.c_raw)
+                store_via_lds([&](int mt, int nt, int vg) {
+                    u32x2 w;
+                    w[0] = E::pack(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
+                    w[1] = E::pack(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
+                    return w;
+                }, p.c_raw + (Cz - pr.C));
+            store_via_lds([&](int mt, int nt, int vg) {
+                const int n = 32 * (WN * wn + nt) + 8 * vg + 4 * g;       // n0 is a multiple of 128
+                const u32x2 wt = *reinterpret_cast<const u32x2*>(p.norm_w + (n & 127));
+                const float r = rr[mt];
+                const u32x2 h = {E::pack(acc[nt][mt][4 * vg] * r, acc[nt][mt][4 * vg + 1] * r),
+                                 E::pack(acc[nt][mt][4 * vg + 2] * r, acc[nt][mt][4 * vg + 3] * r)};
+                u32x2 y;
+                y[0] = E::pack(E::lo(wt[0]) * E::lo(h[0]), E::hi(wt[0]) * E::hi(h[0]));
+                y[1] = E::pack(E::lo(wt[1]) * E::lo(h[1]), E::hi(wt[1]) * E::hi(h[1]));
+                return y;
+            }, Cz);
+            return;
+        }
 #pragma unroll
         for (int mt = 0; mt < WM; ++mt) {
             const int m = m0 + 32 * (WM * wm + mt) + l32;
@@ -396,6 +454,15 @@ epilogue:
                     }
                 }
         }
+        return;
+    }
+    if (VIA_LDS && (p.N & 7) == 0) {
+        store_via_lds([&](int mt, int nt, int vg) {
+            u32x2 w;
+            w[0] = E::pack(acc[nt][mt][4 * vg], acc[nt][mt][4 * vg + 1]);
+            w[1] = E::pack(acc[nt][mt][4 * vg + 2], acc[nt][mt][4 * vg + 3]);
+            return w;
+        }, Cz);
         return;
     }
 #pragma unroll
