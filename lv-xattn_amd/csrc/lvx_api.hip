@@ -572,19 +572,19 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     hipError_t e = launch_bwd(p, s->kv_start != nullptr, st);
     if (e != hipSuccess) return static_cast<int>(e);
     if (scratch) {
-        for (int i = 0; i < 2; ++i) {
-            const lvx_tensor* t = i ? dv : dk;
-            // scratch memory order is [B, Lkv, Hkv, D]: cast with (H, L) = (Lkv, Hkv)
-            CastParams cp{};
-            cp.f16 = p.f16;
-            cp.D = s->D;
-            cp.src = scratch + i * dkv_elems;
-            cp.dst = static_cast<uint16_t*>(t->ptr);
-            cp.ds = Strides3{t->stride_b, t->stride_s, t->stride_h};
-            cp.B = s->B; cp.H = s->Lkv; cp.L = s->Hkv;
-            e = launch_cast(cp, st);
-            if (e != hipSuccess) return static_cast<int>(e);
-        }
+        // scratch memory order is [B, Lkv, Hkv, D]: cast with (H, L) = (Lkv, Hkv); dK and dV in one launch
+        CastParams cp{};
+        cp.f16 = p.f16;
+        cp.D = s->D;
+        cp.src = scratch;
+        cp.dst = static_cast<uint16_t*>(dk->ptr);
+        cp.ds = Strides3{dk->stride_b, dk->stride_s, dk->stride_h};
+        cp.src2 = scratch + dkv_elems;
+        cp.dst2 = static_cast<uint16_t*>(dv->ptr);
+        cp.ds2 = Strides3{dv->stride_b, dv->stride_s, dv->stride_h};
+        cp.B = s->B; cp.H = s->Lkv; cp.L = s->Hkv;
+        e = launch_cast(cp, st);
+        if (e != hipSuccess) return static_cast<int>(e);
     }
 
     // dQ[b, h, rows, :] = dS^T[b, h]^T (rows x tokens) * K[b, h / G] (tokens x D), scale already in dS

@@ -338,35 +338,43 @@ epilogue:
         return;
     }
     // A lane holds 4 consecutive columns of one C row, so storing from the registers writes 8
-    // bytes per lane into 32 different rows per instruction.  Where the tile fits the stage
-    // buffers (free by now) it goes through LDS instead and leaves as whole 512-byte row
-    // segments, 16 bytes per lane.  16-byte chunk c of row r sits at position c ^ (r & 31), with
-    // its two 8-byte halves exchanged in rows where bits 3 and 4 differ: the 32 rows a half-wave's
-    // 8-byte writes touch then land in 32 different chunks, and those of them that share banks
-    // (positions 8 or 16 apart) in different halves; a read instruction takes the 32 chunks of two
-    // rows.  Both are conflict-free.  `pair(mt, nt, vg)`: the 4 values of accumulator tile (nt, mt), register
-    // group vg, as two packed words.
-    constexpr bool VIA_LDS = TN == 256 && TM * TN * 2 <= NS * STAGE;
+    // bytes per lane into 32 different rows per instruction.  Where 256 rows of the tile fit the
+    // stage buffers (free by now) they go through LDS instead, 256 rows at a time, and leave as
+    // whole row segments (TN * 2 bytes), 16 bytes per lane.  16-byte chunk c of row r sits at
+    // position c ^ (r mod chunks per row), with its two 8-byte halves exchanged in rows where
+    // bits 3 and 4 differ: the 32 rows a half-wave's 8-byte writes touch then land in different
+    // chunks or, where they share a chunk position or banks (positions 8 or 16 apart), in
+    // different halves; a read instruction takes whole rows.  Both are conflict-free.
+    // `pair(mt, nt, vg)`: the 4 values of accumulator tile (nt, mt), register group vg, as two
+    // packed words.
+    constexpr int CPR = TN / 8;                 // 16-byte chunks per row
+    constexpr bool VIA_LDS = (TN == 256 || TN == 128) && TM % 256 == 0 && 256 * TN * 2 <= NS * STAGE;
     auto store_via_lds = [&](auto pair, uint16_t* dst) __attribute__((always_inline)) {
-        __syncthreads();                    // every wave is done with what the buffers held
 #pragma unroll
-        for (int mt = 0; mt < WM; ++mt)
+        for (int pass = 0; pass < TM / 256; ++pass) {
+            __syncthreads();                    // every wave is done with what the buffers held
 #pragma unroll
-            for (int nt = 0; nt < WN; ++nt)
+            for (int mt = 0; mt < WM; ++mt) {
+                if (((WM * wm + mt) >> 3) != pass) continue;
 #pragma unroll
-                for (int vg = 0; vg < 4; ++vg) {
-                    const int ml = 32 * (WM * wm + mt) + l32;
-                    const int c = 4 * (WN * wn + nt) + vg;
-                    *reinterpret_cast<u32x2*>(lds + ml * (TN * 2) + ((c ^ l32) << 4) + ((g ^ ((l32 >> 3) & 1) ^ (l32 >> 4)) << 3)) = pair(mt, nt, vg);
-                }
-        __syncthreads();
+                for (int nt = 0; nt < WN; ++nt)
 #pragma unroll
-        for (int i = 0; i < TM / 16; ++i) {
-            const int row = i * 16 + (tid >> 5), cc = tid & 31;
-            u32x4 val = *reinterpret_cast<const u32x4*>(lds + row * (TN * 2) + ((cc ^ (row & 31)) << 4));
-            if (((row >> 3) ^ (row >> 4)) & 1) val = u32x4{val[2], val[3], val[0], val[1]};
-            const int m = m0 + row, n = n0 + cc * 8;
-            if (m < p.M && n < p.N) *reinterpret_cast<u32x4*>(dst + (int64_t)m * pr.ldc + n) = val;
+                    for (int vg = 0; vg < 4; ++vg) {
+                        const int ml = 32 * ((WM * wm + mt) & 7) + l32;
+                        const int c = 4 * (WN * wn + nt) + vg;
+                        *reinterpret_cast<u32x2*>(lds + ml * (TN * 2) + ((c ^ (l32 & (CPR - 1))) << 4) +
+                                                  ((g ^ ((l32 >> 3) & 1) ^ (l32 >> 4)) << 3)) = pair(mt, nt, vg);
+                    }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < CPR / 2; ++i) {
+                const int row = i * (512 / CPR) + tid / CPR, cc = tid % CPR;
+                u32x4 val = *reinterpret_cast<const u32x4*>(lds + row * (TN * 2) + ((cc ^ (row & (CPR - 1))) << 4));
+                if (((row >> 3) ^ (row >> 4)) & 1) val = u32x4{val[2], val[3], val[0], val[1]};
+                const int m = m0 + 256 * pass + row, n = n0 + cc * 8;
+                if (m < p.M && n < p.N) *reinterpret_cast<u32x4*>(dst + (int64_t)m * pr.ldc + n) = val;
+            }
         }
     };
     if (p.norm_w && t2 / p.nbatch == 0) {

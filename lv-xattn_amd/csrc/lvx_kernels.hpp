@@ -159,6 +159,10 @@ struct CastParams {
     const float* src;
     uint16_t* dst;
     Strides3 ds;
+    // a second tensor of the same sizes, cast by the same launch (null: none)
+    const float* src2;
+    uint16_t* dst2;
+    Strides3 ds2;
     int B, H, L;
     int transposed;   // 0: src is [B*H][L][D]; 1: src is [B*H][D][L]
     int nsum;         // transposed only: the result is the sum of nsum such sources (0 or 1: one),

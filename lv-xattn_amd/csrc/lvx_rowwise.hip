@@ -357,14 +357,16 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     const int row = (int)(r % p.L);
     const int bh = (int)(r / p.L);
     const int b = bh / p.H, h = bh % p.H;
-    const f32x4* s = reinterpret_cast<const f32x4*>(p.src + r * Dh + chunk * 8);
+    const bool second = blockIdx.y != 0;
+    const f32x4* s = reinterpret_cast<const f32x4*>((second ? p.src2 : p.src) + r * Dh + chunk * 8);
     const f32x4 a = s[0], c = s[1];
     u32x4 u;
     u[0] = E::pack(a[0], a[1]);
     u[1] = E::pack(a[2], a[3]);
     u[2] = E::pack(c[0], c[1]);
     u[3] = E::pack(c[2], c[3]);
-    *reinterpret_cast<u32x4*>(p.dst + b * p.ds.b + h * p.ds.h + (int64_t)row * p.ds.s + chunk * 8) = u;
+    const Strides3 ds = second ? p.ds2 : p.ds;
+    *reinterpret_cast<u32x4*>((second ? p.dst2 : p.dst) + b * ds.b + h * ds.h + (int64_t)row * ds.s + chunk * 8) = u;
 }
 
 // Same from a transposed source [B*H][D][L], or the sum of several: adjacent threads take
@@ -517,8 +519,9 @@ hipError_t launch_norm_bwd(const NormBwdParams& p, hipStream_t st) {
 hipError_t launch_cast(const CastParams& p, hipStream_t st) {
     const int64_t rows = (int64_t)p.B * p.H * p.L;
     if (rows == 0) return hipSuccess;
-    const dim3 grid(blocks_for(rows));
+    const dim3 grid(blocks_for(rows), !p.transposed && p.src2 ? 2 : 1);
     if (p.transposed) {
+        if (p.src2) return hipErrorInvalidValue;
         if (p.f16) return launch1(cast_t_kernel<true>, grid, dim3(256), st, p);
         else return launch1(cast_t_kernel<false>, grid, dim3(256), st, p);
     } else {
