@@ -29,7 +29,7 @@ ROUND_STREAMS = 4            # streams the one-launch-per-round mode may spread 
 
 
 def bwd_traffic_bytes(name):
-    """HBM bytes moved by one lvx_bwd call (metadata + dK/dV kernel + 2 casts + dQ GEMM) as
+    """HBM bytes moved by one lvx_bwd call (metadata + dK/dV kernel + cast + dQ GEMM) as
     the counter summary of that workload states them (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
     runs scaled by a 1 GiB copy): the `traffic_bytes_per_call:` line of
     profiles/<name>_bwd_hbm_traffic.md.  None when there is no such summary."""
@@ -508,7 +508,7 @@ def main():
         kb = kernel_breakdown(layer, npairs, torch)
         out["kernels"] = kb
         dom = kb["bwd_all_rounds_one_launch"]
-        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel (incl. scratch zero-fill) + bwd_kernel + 2 cast_kernel + dQ gemm_kernel",
+        out["roofline"] = {"bound": "mfma", "kernel": "lvx_bwd = bwd_meta_kernel (incl. scratch zero-fill) + bwd_kernel + cast_kernel + dQ gemm_kernel",
                            "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(dom["tflops"] / PEAK_BF16_TFLOPS, 4),
                            "traffic": bwd_traffic_bytes(w.name) if a.mode == "batched" else None,
