@@ -393,9 +393,18 @@ static int cu_count() {
     return n;
 }
 
-static int choose_q_splits(int blocks, int steps, bool masked) {
+// How the token blocks of a launch are handed to work-groups (see bwd_kernel): per XCD, the first
+// `whole` blocks get one work-group each and the others `splits` work-groups each.
+struct BwdCut {
+    int blocks_per_xcd, whole, splits;
+};
+
+static BwdCut choose_bwd_cut(int blocks, int steps, bool masked) {
     constexpr double WG_COST = 6.0, SPLIT_COST = 55.0;
+    constexpr int XCDS = 8;
     const int n_cu = cu_count();
+    BwdCut cut;
+    cut.blocks_per_xcd = (blocks + XCDS - 1) / XCDS;
     // unequal work-groups only even out when there are enough of them; a small masked launch
     // is priced like a dense one (which is also right when its mask hides nothing)
     const bool ragged = masked && blocks >= 2 * n_cu;
@@ -412,7 +421,22 @@ static int choose_q_splits(int blocks, int steps, bool masked) {
         const double c = cost(S);
         if (c < best_cost) { best_cost = c; best = S; }
     }
-    return best;
+    cut.splits = best;
+    cut.whole = best == 1 ? cut.blocks_per_xcd : 0;
+    // Equal blocks, more of them than CUs: whole rounds of unsplit blocks first (no partial sums,
+    // one ramp per block), and only the blocks past the last whole round are cut, into as many
+    // ranges as fill their rounds best.
+    const int cu_x = n_cu / XCDS;
+    if (!ragged && cu_x > 0 && cut.blocks_per_xcd > cu_x && blocks % XCDS == 0) {
+        const int full = cut.blocks_per_xcd / cu_x * cu_x, rest = cut.blocks_per_xcd - full;
+        if (rest == 0) return cut;       // (best is 1 then)
+        for (int S = 2; S <= 8; ++S) {
+            if (steps / S < 32) break;
+            const double c = (full / cu_x) * (steps + WG_COST) + ((rest * S + cu_x - 1) / cu_x) * ((double)steps / S + WG_COST) + SPLIT_COST;
+            if (c < best_cost) { best_cost = c; cut.splits = S; cut.whole = full; }
+        }
+    }
+    return cut;
 }
 
 static size_t dkv_scratch_bytes(const lvx_attn_shape* s) {
@@ -528,9 +552,11 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     // metadata kernel zeroes them on its way
     const int blocks = s->B * s->Hkv * p.n_kv_blocks;
     const int steps = p.G * (int)(rows / 32);
-    p.q_splits = choose_q_splits(blocks, steps, s->kv_start != nullptr);
-    p.split_steps = (steps + p.q_splits - 1) / p.q_splits;
-    p.total_wg = blocks * p.q_splits;
+    const BwdCut cut = choose_bwd_cut(blocks, steps, s->kv_start != nullptr);
+    p.n_blocks = blocks;
+    p.blocks_per_xcd = cut.blocks_per_xcd;
+    p.whole_blocks = cut.whole;
+    p.q_splits = cut.splits;
     p.dkv_mode = p.q_splits > 1 ? 2 : (dkv_accumulate ? 1 : 0);
     float* const scratch = (p.q_splits > 1 && !dkv_accumulate) ? reinterpret_cast<float*>(wsb + wsl.dkv) : nullptr;
     int split_len = 0;

@@ -88,11 +88,28 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // LSE*log2e, delta*scale, kv_start, kv_end
     __shared__ __attribute__((aligned(256))) u32x4 meta_s4[NQD][BM];
 
-    const int wid = xcd_remap(blockIdx.x, p.total_wg);
-    if (wid >= p.total_wg) return;
-    const int sp = wid % p.q_splits;
-    const int kblk = (wid / p.q_splits) % p.n_kv_blocks;
-    const int bh = wid / (p.q_splits * p.n_kv_blocks);
+    // Work-group ids are dealt to the 8 XCDs round-robin.  XCD x takes the token blocks
+    // [x * blocks_per_xcd, (x + 1) * blocks_per_xcd) of the list (b, kv head, block), so that the
+    // work-groups of a kv head share an L2: first `whole_blocks` of them with one work-group
+    // each, then the others with q_splits work-groups each, the longer work-groups first.  (A
+    // placement hint only: every (block, range) is produced exactly once whatever the hardware
+    // does with the ids.)
+    const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
+    const int blk0 = xcd * p.blocks_per_xcd;
+    const int nblk = min(p.blocks_per_xcd, p.n_blocks - blk0);
+    const int whole = max(0, min(p.whole_blocks, nblk));
+    int blk, sp = 0, S = 1;
+    if (local < whole) {
+        blk = blk0 + local;
+    } else {
+        const int l2 = local - whole;
+        S = p.q_splits;
+        sp = l2 % S;
+        blk = blk0 + whole + l2 / S;
+        if (blk >= blk0 + nblk) return;
+    }
+    const int kblk = blk % p.n_kv_blocks;
+    const int bh = blk / p.n_kv_blocks;
     const int b = bh % p.B;            // samples interleaved: ragged samples then share the tail of the launch
     const int hk = bh / p.B;
 
@@ -116,7 +133,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // with an interval mask only the listed runs of tiles are visited (kept in scalar
     // registers), and the splits share that shorter walk evenly
     int run_s[4] = {0, 0, 0, 0}, run_n[4] = {n_qtiles, 0, 0, 0};
-    int n_live = n_qtiles, split_steps = p.split_steps;
+    int n_live = n_qtiles;
     if (MASKED && p.live_runs) {
         const int32_t* lr = p.live_runs + ((int64_t)b * p.n_kv_blocks + kblk) * 8;
 #pragma unroll
@@ -125,8 +142,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             run_n[i] = __builtin_amdgcn_readfirstlane(lr[2 * i + 1]);
         }
         n_live = run_n[0] + run_n[1] + run_n[2] + run_n[3];
-        split_steps = (p.G * n_live + p.q_splits - 1) / p.q_splits;
     }
+    const int split_steps = (p.G * n_live + S - 1) / S;
     auto sel4 = [](int r, const int (&a)[4]) { return r == 0 ? a[0] : r == 1 ? a[1] : r == 2 ? a[2] : a[3]; };
     const int it_lo = sp * split_steps;
     const int n_iter = (kvb < kv_len) ? max(0, min(split_steps, p.G * n_live - it_lo)) : 0;
@@ -652,7 +669,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 namespace {
 template <int DH, bool F16>
 hipError_t launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
-    const int grid = ((p.total_wg + 7) / 8) * 8;
+    const int grid = 8 * (p.whole_blocks + (p.blocks_per_xcd - p.whole_blocks) * p.q_splits);
     if (p.bias) {
         if (masked) return launch1((bwd_kernel<DH, true, true, F16>), dim3(grid), dim3(NT), st, p);
         else return launch1((bwd_kernel<DH, false, true, F16>), dim3(grid), dim3(NT), st, p);

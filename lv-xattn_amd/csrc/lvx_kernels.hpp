@@ -110,9 +110,11 @@ struct BwdParams {
     int B, Hq, Hkv, Lq, Lkv, G;
     int D;                     // head dimension: 16, 32, 64 or 128
     int row_begin, row_end;
-    int n_kv_blocks, total_wg;
-    int q_splits;              // work-groups sharing one token block, each taking a range of steps
-    int split_steps;           // steps (32-row tiles x heads of the group) per split
+    int n_kv_blocks;
+    int n_blocks;              // token blocks of all (b, kv head): B * Hkv * n_kv_blocks
+    int blocks_per_xcd;        // ceil(n_blocks / 8): the token blocks an XCD's work-groups take
+    int whole_blocks;          // of an XCD's blocks, the first so many get one work-group each (0 .. blocks_per_xcd)
+    int q_splits;              // work-groups sharing each of the other blocks, each taking a range of steps
     int dkv_mode;              // 0: store bf16, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1)
     float scale, scale_log2e;
     // Interval masks: the 32-row tiles each token block has to visit (the others see none of
