@@ -588,9 +588,13 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     }
 
     const int64_t dkv_elems = (int64_t)s->B * s->Lkv * s->Hkv * s->D;
+    // blocks with one work-group are written by it as the caller asked
+    p.dk_whole = p.dk; p.dv_whole = p.dv;
+    p.dks_whole = p.dks; p.dvs_whole = p.dvs;
+    p.whole_mode = dkv_accumulate ? 1 : 0;
     if (scratch) {
-        // bf16 outputs, several work-groups per token block: sum in the fp32 scratch
-        // [2][B, Lkv, Hkv, D], round once afterwards
+        // bf16 outputs, several work-groups per token block: those blocks are summed in the fp32
+        // scratch [2][B, Lkv, Hkv, D] and rounded once afterwards
         p.dk = scratch;
         p.dv = scratch + dkv_elems;
         p.dks = p.dvs = Strides3{(int64_t)s->Lkv * s->Hkv * s->D, (int64_t)s->D, (int64_t)s->Hkv * s->D};
@@ -609,6 +613,10 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
         cp.dst2 = static_cast<uint16_t*>(dv->ptr);
         cp.ds2 = Strides3{dv->stride_b, dv->stride_s, dv->stride_h};
         cp.B = s->B; cp.H = s->Lkv; cp.L = s->Hkv;
+        if (p.whole_blocks > 0) {
+            cp.skip_bpx = p.blocks_per_xcd; cp.skip_whole = p.whole_blocks;
+            cp.skip_nkvb = p.n_kv_blocks; cp.skip_nblocks = p.n_blocks;
+        }
         e = launch_cast(cp, st);
         if (e != hipSuccess) return static_cast<int>(e);
     }

@@ -148,7 +148,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     const int it_lo = sp * split_steps;
     const int n_iter = (kvb < kv_len) ? max(0, min(split_steps, p.G * n_live - it_lo)) : 0;
     // nothing to visit and nothing to overwrite: done (bf16 outputs, mode 0, still get their zeros)
-    if (n_iter == 0 && p.dkv_mode != 0) return;
+    // a block that its work-group owns alone is written by it directly, also when others are shared
+    const bool alone = p.dkv_mode == 2 && S == 1;
+    const int dkv_mode = alone ? p.whole_mode : p.dkv_mode;
+    if (n_iter == 0 && dkv_mode != 0) return;
 
     // ---- resident B operand: this wave's K rows (P-wave) or V rows (D-wave)
     bf16x8 breg[8];     // [NKK .. 8) stay unused when DH < 128
@@ -607,7 +610,7 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     }
 
     // ---- epilogue: rows of acc = head-dim, cols = this wave's tokens; P-waves hold dV^T, D-waves dK^T
-    if (p.dkv_mode == 2) {
+    if (dkv_mode == 2) {
         // Several work-groups (ranges of steps) share this token block: add with
         // atomics.  The accumulator has tokens along the lanes; it is turned
         // through LDS so that each atomic instruction covers 64 consecutive
@@ -631,10 +634,10 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
             }
         }
     } else if (my_kv < p.Lkv) {
-        const Strides3 os = d_role ? p.dks : p.dvs;
-        void* optr = d_role ? p.dk : p.dv;
+        const Strides3 os = alone ? (d_role ? p.dks_whole : p.dvs_whole) : (d_role ? p.dks : p.dvs);
+        void* optr = alone ? (d_role ? p.dk_whole : p.dv_whole) : (d_role ? p.dk : p.dv);
         const int64_t off = b * os.b + hk * os.h + (int64_t)my_kv * os.s;
-        if (p.dkv_mode == 1) {
+        if (dkv_mode == 1) {
             float* op = reinterpret_cast<float*>(optr) + off;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)

@@ -115,7 +115,12 @@ struct BwdParams {
     int blocks_per_xcd;        // ceil(n_blocks / 8): the token blocks an XCD's work-groups take
     int whole_blocks;          // of an XCD's blocks, the first so many get one work-group each (0 .. blocks_per_xcd)
     int q_splits;              // work-groups sharing each of the other blocks, each taking a range of steps
-    int dkv_mode;              // 0: store bf16, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1)
+    int dkv_mode;              // 0: store 16-bit, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1: the shared blocks)
+    // mode 2: where and how the work-group of a block it owns alone writes (whole_mode 0 or 1)
+    void* dk_whole;
+    void* dv_whole;
+    Strides3 dks_whole, dvs_whole;
+    int whole_mode;
     float scale, scale_log2e;
     // Interval masks: the 32-row tiles each token block has to visit (the others see none of
     // its tokens) as up to 4 runs of consecutive tiles, live_runs[(b * n_kv_blocks + block) * 8
@@ -165,6 +170,10 @@ struct CastParams {
     const float* src2;
     uint16_t* dst2;
     Strides3 ds2;
+    // the fp32 dK / dV scratch of the backward, (H, L) = (tokens, kv heads): rows of token blocks that
+    // the kernel wrote directly (the first skip_whole of every skip_bpx blocks of the list (b, kv
+    // head, block), skip_nkvb blocks per (b, kv head), skip_nblocks in all) are left alone.  skip_bpx 0: none.
+    int skip_bpx, skip_whole, skip_nkvb, skip_nblocks;
     int B, H, L;
     int transposed;   // 0: src is [B*H][L][D]; 1: src is [B*H][D][L]
     int nsum;         // transposed only: the result is the sum of nsum such sources (0 or 1: one),

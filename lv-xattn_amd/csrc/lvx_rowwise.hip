@@ -357,6 +357,11 @@ __global__ __launch_bounds__(256) void cast_kernel(const CastParams p) {
     const int row = (int)(r % p.L);
     const int bh = (int)(r / p.L);
     const int b = bh / p.H, h = bh % p.H;
+    if (p.skip_bpx) {      // h is a token, row a kv head
+        const int blk = (h >> 7) + p.skip_nkvb * (b + p.B * row);
+        const int first = blk / p.skip_bpx * p.skip_bpx;
+        if (blk - first < min(p.skip_whole, p.skip_nblocks - first)) return;
+    }
     const bool second = blockIdx.y != 0;
     const f32x4* s = reinterpret_cast<const f32x4*>((second ? p.src2 : p.src) + r * Dh + chunk * 8);
     const f32x4 a = s[0], c = s[1];
