@@ -394,17 +394,20 @@ static int cu_count() {
 }
 
 // How the token blocks of a launch are handed to work-groups (see bwd_kernel): per XCD, the first
-// `whole` blocks get one work-group each and the others `splits` work-groups each.
+// `whole` blocks get one work-group each, the next `mid` blocks `splits` work-groups each and the
+// others `splits2` each.
 struct BwdCut {
-    int blocks_per_xcd, whole, splits;
+    int blocks_per_xcd, whole, mid, splits, splits2;
+    bool any_split() const { return (mid > 0 && splits > 1) || (whole + mid < blocks_per_xcd && splits2 > 1); }
 };
 
 static BwdCut choose_bwd_cut(int blocks, int steps, bool masked) {
     constexpr double WG_COST = 6.0, SPLIT_COST = 55.0;
-    constexpr int XCDS = 8;
+    constexpr int XCDS = 8, MAX_SPLITS_PER_BLOCK = 16, MIN_RANGE = 32;
     const int n_cu = cu_count();
     BwdCut cut;
     cut.blocks_per_xcd = (blocks + XCDS - 1) / XCDS;
+    cut.splits2 = 1;
     // unequal work-groups only even out when there are enough of them; a small masked launch
     // is priced like a dense one (which is also right when its mask hides nothing)
     const bool ragged = masked && blocks >= 2 * n_cu;
@@ -417,23 +420,36 @@ static BwdCut choose_bwd_cut(int blocks, int steps, bool masked) {
     int best = 1;
     double best_cost = cost(1);
     for (int S = 2; S <= 8; ++S) {
-        if (steps / S < 32) break;
+        if (steps / S < MIN_RANGE) break;
         const double c = cost(S);
         if (c < best_cost) { best_cost = c; best = S; }
     }
     cut.splits = best;
     cut.whole = best == 1 ? cut.blocks_per_xcd : 0;
+    cut.mid = cut.blocks_per_xcd - cut.whole;
     // Equal blocks, more of them than CUs: whole rounds of unsplit blocks first (no partial sums,
-    // one ramp per block), and only the blocks past the last whole round are cut, into as many
-    // ranges as fill their rounds best.
+    // one ramp per block), and only the blocks past the last whole round are cut - all alike into
+    // as many ranges as fill their rounds best, or in two groups that make one round each: as
+    // many blocks as give every CU one work-group when cut in S1 = ceil(CUs / blocks), and what
+    // is left then in as many ranges as the CUs can take.
     const int cu_x = n_cu / XCDS;
     if (!ragged && cu_x > 0 && cut.blocks_per_xcd > cu_x && blocks % XCDS == 0) {
         const int full = cut.blocks_per_xcd / cu_x * cu_x, rest = cut.blocks_per_xcd - full;
         if (rest == 0) return cut;       // (best is 1 then)
+        const double whole_cost = (full / cu_x) * (steps + WG_COST) + SPLIT_COST;
         for (int S = 2; S <= 8; ++S) {
-            if (steps / S < 32) break;
-            const double c = (full / cu_x) * (steps + WG_COST) + ((rest * S + cu_x - 1) / cu_x) * ((double)steps / S + WG_COST) + SPLIT_COST;
-            if (c < best_cost) { best_cost = c; cut.splits = S; cut.whole = full; }
+            if (steps / S < MIN_RANGE) break;
+            const double c = whole_cost + ((rest * S + cu_x - 1) / cu_x) * ((double)steps / S + WG_COST);
+            if (c < best_cost) { best_cost = c; cut.whole = full; cut.mid = rest; cut.splits = S; cut.splits2 = 1; }
+        }
+        const int S1 = (cu_x + rest - 1) / rest;
+        const int n1 = std::min(rest, cu_x / S1), left = rest - n1;
+        if (S1 >= 2 && steps / S1 >= MIN_RANGE && left > 0) {
+            int S2 = std::min(std::min(cu_x / left, MAX_SPLITS_PER_BLOCK), steps / MIN_RANGE);
+            if (S2 >= 2) {
+                const double c = whole_cost + ((double)steps / S1 + WG_COST) + ((double)steps / S2 + WG_COST);
+                if (c < best_cost) { best_cost = c; cut.whole = full; cut.mid = n1; cut.splits = S1; cut.splits2 = S2; }
+            }
         }
     }
     return cut;
@@ -556,9 +572,11 @@ int lvx_bwd(const lvx_attn_shape* s, const lvx_tensor* q, const lvx_tensor* k, c
     p.n_blocks = blocks;
     p.blocks_per_xcd = cut.blocks_per_xcd;
     p.whole_blocks = cut.whole;
+    p.mid_blocks = cut.mid;
     p.q_splits = cut.splits;
-    p.dkv_mode = p.q_splits > 1 ? 2 : (dkv_accumulate ? 1 : 0);
-    float* const scratch = (p.q_splits > 1 && !dkv_accumulate) ? reinterpret_cast<float*>(wsb + wsl.dkv) : nullptr;
+    p.q_splits2 = cut.splits2;
+    p.dkv_mode = cut.any_split() ? 2 : (dkv_accumulate ? 1 : 0);
+    float* const scratch = (cut.any_split() && !dkv_accumulate) ? reinterpret_cast<float*>(wsb + wsl.dkv) : nullptr;
     int split_len = 0;
     const int ks = dq_k_splits(s, row_count, &split_len);
     float* const dq32 = ks > 1 ? reinterpret_cast<float*>(wsb + wsl.dq32) : nullptr;

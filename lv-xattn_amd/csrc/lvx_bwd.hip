@@ -91,21 +91,27 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
     // Work-group ids are dealt to the 8 XCDs round-robin.  XCD x takes the token blocks
     // [x * blocks_per_xcd, (x + 1) * blocks_per_xcd) of the list (b, kv head, block), so that the
     // work-groups of a kv head share an L2: first `whole_blocks` of them with one work-group
-    // each, then the others with q_splits work-groups each, the longer work-groups first.  (A
-    // placement hint only: every (block, range) is produced exactly once whatever the hardware
-    // does with the ids.)
+    // each, then `mid_blocks` with q_splits work-groups each, then the others with q_splits2
+    // each - the longer work-groups first.  (A placement hint only: every (block, range) is
+    // produced exactly once whatever the hardware does with the ids.)
     const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
     const int blk0 = xcd * p.blocks_per_xcd;
     const int nblk = min(p.blocks_per_xcd, p.n_blocks - blk0);
     const int whole = max(0, min(p.whole_blocks, nblk));
+    const int mid = max(0, min(p.mid_blocks, nblk - whole));
     int blk, sp = 0, S = 1;
     if (local < whole) {
         blk = blk0 + local;
-    } else {
+    } else if (local < whole + mid * p.q_splits) {
         const int l2 = local - whole;
         S = p.q_splits;
         sp = l2 % S;
         blk = blk0 + whole + l2 / S;
+    } else {
+        const int l3 = local - whole - mid * p.q_splits;
+        S = p.q_splits2;
+        sp = l3 % S;
+        blk = blk0 + whole + mid + l3 / S;
         if (blk >= blk0 + nblk) return;
     }
     const int kblk = blk % p.n_kv_blocks;
@@ -672,7 +678,8 @@ __global__ __launch_bounds__(NT, 1) void bwd_kernel(const BwdParams p) {
 namespace {
 template <int DH, bool F16>
 hipError_t launch_bwd_t(const BwdParams& p, bool masked, hipStream_t st) {
-    const int grid = 8 * (p.whole_blocks + (p.blocks_per_xcd - p.whole_blocks) * p.q_splits);
+    const int grid = 8 * (p.whole_blocks + p.mid_blocks * p.q_splits +
+                          (p.blocks_per_xcd - p.whole_blocks - p.mid_blocks) * p.q_splits2);
     if (p.bias) {
         if (masked) return launch1((bwd_kernel<DH, true, true, F16>), dim3(grid), dim3(NT), st, p);
         else return launch1((bwd_kernel<DH, false, true, F16>), dim3(grid), dim3(NT), st, p);

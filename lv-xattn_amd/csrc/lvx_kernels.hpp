@@ -113,8 +113,9 @@ struct BwdParams {
     int n_kv_blocks;
     int n_blocks;              // token blocks of all (b, kv head): B * Hkv * n_kv_blocks
     int blocks_per_xcd;        // ceil(n_blocks / 8): the token blocks an XCD's work-groups take
-    int whole_blocks;          // of an XCD's blocks, the first so many get one work-group each (0 .. blocks_per_xcd)
-    int q_splits;              // work-groups sharing each of the other blocks, each taking a range of steps
+    int whole_blocks;          // of an XCD's blocks, the first so many get one work-group each (0 .. blocks_per_xcd),
+    int mid_blocks, q_splits;  // the next mid_blocks are shared by q_splits work-groups each, every one taking a range of steps,
+    int q_splits2;             // and the others by q_splits2 (>= 1) work-groups each
     int dkv_mode;              // 0: store 16-bit, 1: fp32 +=, 2: fp32 atomic += (q_splits > 1: the shared blocks)
     // mode 2: where and how the work-group of a block it owns alone writes (whole_mode 0 or 1)
     void* dk_whole;
