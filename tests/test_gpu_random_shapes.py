@@ -256,3 +256,15 @@ def test_row_groups_with_hulls_of_many_lengths(lvx, seed):
     check_grad(dv, dv_ref, "dV")
     dead = torch.isinf(l_ref).reshape(B, Hq, Lq)
     assert (dq.float().cpu()[dead] == 0).all()
+
+
+@pytest.mark.parametrize("Lq,D", [(8192, 16), (2048, 64)])
+def test_backward_blocks_cut_in_groups(lvx, Lq, D):
+    # 8 kv heads x 51 token blocks on a 256-CU GPU are 51 blocks per XCD of 32 CUs.  With 256 steps
+    # per block (8192 rows) 32 of them get a work-group each and are written directly, and the 19
+    # past the whole round are cut into row ranges (16 blocks in two, 3 in eight) whose partial
+    # dK / dV are added in the fp32 scratch and cast: both kinds of block in one launch.  With 64
+    # steps per block no cut pays and the launch is two rounds of whole blocks.
+    rng = random.Random(77)
+    g = torch.Generator().manual_seed(78)
+    _run_case(lvx, 1, 8, 8, Lq, 6404, 1, True, "none", rng, g, strided=False, sigma=0.5, D=D)
