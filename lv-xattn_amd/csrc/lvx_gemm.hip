@@ -373,7 +373,8 @@ epilogue:
                 u32x4 val = *reinterpret_cast<const u32x4*>(lds + row * (TN * 2) + ((cc ^ (row & (CPR - 1))) << 4));
                 if (((row >> 3) ^ (row >> 4)) & 1) val = u32x4{val[2], val[3], val[0], val[1]};
                 const int m = m0 + 256 * pass + row, n = n0 + cc * 8;
-                if (m < p.M && n < p.N) *reinterpret_cast<u32x4*>(dst + (int64_t)m * pr.ldc + n) = val;
+                // (a streaming store: nobody on this CU reads the tile again)
+                if (m < p.M && n < p.N) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst + (int64_t)m * pr.ldc + n));
             }
         }
     };
